@@ -45,6 +45,8 @@ class _Group:
     page_size: int
     window: int | None
     chunk: int | None = None
+    # a window group keeps the pages of the sequence's first `keep_first` positions for good
+    keep_first: int = 0
     tables: dict[Hashable, list[int]] = field(default_factory=dict)
     # index of the first table entry that still holds a page
     first_live: dict[Hashable, int] = field(default_factory=dict)
@@ -86,7 +88,8 @@ class CacheManager:
             if spec.paged:
                 key = spec.group_key()
                 if key not in by_key:
-                    by_key[key] = _Group(key, spec, [], PagePool(num_pages), self.page_size, spec.window, spec.chunk)
+                    by_key[key] = _Group(key, spec, [], PagePool(num_pages), self.page_size, spec.window, spec.chunk,
+                                         spec.keep_first)
                     self.groups.append(by_key[key])
                 by_key[key].cache_ids.append(cid)
                 self._group_of_cache[cid] = self.groups.index(by_key[key])
@@ -131,7 +134,7 @@ class CacheManager:
     def _visible(spec: CacheSpec, length: int) -> int:
         """Keys that the newest of ``length`` tokens sees in a cache of ``spec``."""
         if spec.window is not None:
-            return min(length, spec.window)
+            return min(length, spec.window + spec.keep_first)
         if spec.chunk is not None and length > 0:
             return (length - 1) % spec.chunk + 1
         return length
@@ -156,7 +159,7 @@ class CacheManager:
             need = g.pages_for(length)
             if g.window is not None:
                 # `window` consecutive positions touch at most this many pages
-                need = min(need, (g.window - 1 + g.page_size - 1) // g.page_size + 1)
+                need = min(need, (g.window - 1 + g.page_size - 1) // g.page_size + 1 + g.pages_for(g.keep_first))
             if g.chunk is not None:
                 # a chunk's positions likewise (it need not begin where a page begins)
                 need = min(need, (g.chunk - 1 + g.page_size - 1) // g.page_size + 1)
@@ -251,7 +254,8 @@ class CacheManager:
             else:
                 continue
             table = g.tables[rid]
-            i = g.first_live[rid]
+            # pages that hold any of the first tokens a window keeps in sight are never given back
+            i = max(g.first_live[rid], g.pages_for(g.keep_first))
             while i < len(table) and (i + 1) * g.page_size <= first_needed:
                 g.pool.give(table[i], rid)
                 table[i] = -1

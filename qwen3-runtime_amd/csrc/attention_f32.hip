@@ -7,7 +7,10 @@
 // head h / g. The query at position p sees keys j <= p, and j > p - window when
 // a window is set, or j >= p - p % chunk when a chunk size is. Scores are
 // dot * scale, then, with a cap, cap * tanh(score / cap). Values may have another
-// size Dv than keys; with a gate the output is multiplied by sigmoid(gate). Cache
+// size Dv than keys; with a gate the output is multiplied by sigmoid(gate). Beside a window the
+// first keep_first keys of the sequence stay visible to every later query (their pages stay in the
+// table; the pages between them and the window may be gone and are not touched). With a sink the
+// softmax's denominator has one more term of score 0: p_j = exp(s_j) / (1 + sum exp(s_j)). Cache
 // layout: keys [page, head, offset, D], values [page, head, Dv, offset].
 #include "common.h"
 #include <math.h>
@@ -28,6 +31,8 @@ struct AttnArgs {
   int value_dim;   // 0: head_dim
   const void* gate;  // [T, gate_stride] with nq * Dv columns used, or null
   long gate_stride;
+  int keep_first;  // with a window: keys j < keep_first are seen too
+  int sink;        // 1: one more term exp(0) in the denominator
 };
 
 #define MAX_D 512
@@ -53,9 +58,13 @@ __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
 
   const T* kc = (const T*)a.k_cache;
   const T* vc = (const T*)a.v_cache;
-  for (int j0 = lo; j0 <= pos; j0 += 64) {
+  // two stretches of keys: the kept first ones that lie before the window, then the window
+  const int kept_end = a.window > 0 ? min(a.keep_first, lo) : 0;
+  for (int seg = kept_end > 0 ? 0 : 1; seg < 2; ++seg) {
+  const int seg_begin = seg == 0 ? 0 : lo, seg_last = seg == 0 ? kept_end - 1 : pos;
+  for (int j0 = seg_begin; j0 <= seg_last; j0 += 64) {
     const int j = j0 + lane;
-    const bool valid = j <= pos;
+    const bool valid = j <= seg_last;
     float s = -INFINITY;
     int page = 0, off = 0;
     if (valid) {
@@ -74,7 +83,7 @@ __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
     m = m_new;
 #pragma unroll
     for (int i = 0; i < MAX_D / 64; ++i) acc[i] *= corr;
-    const int n = min(64, pos - j0 + 1);
+    const int n = min(64, seg_last - j0 + 1);
     for (int jj = 0; jj < n; ++jj) {
       const float pj = __shfl(p, jj, 64);
       const int pg = __shfl(page, jj, 64);
@@ -86,6 +95,14 @@ __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
         if (d < Dv) acc[i] = fmaf(pj, to_f32<T>(vr[(size_t)d * ps]), acc[i]);
       }
     }
+  }
+  }
+  if (a.sink) {  // the sink: a key of score 0 without a value
+    const float m_new = fmaxf(m, 0.f);
+    const float corr = expf(m - m_new);
+    l = l * corr + expf(-m_new);
+#pragma unroll
+    for (int i = 0; i < MAX_D / 64; ++i) acc[i] *= corr;
   }
   T* o = (T*)a.out + ((size_t)t * a.nq + h) * Dv;
   const T* gate = a.gate ? (const T*)a.gate + (size_t)t * a.gate_stride + (size_t)h * Dv : nullptr;
@@ -111,6 +128,7 @@ extern "C" int qrt_attention_f32(const AttnArgs* args, int dtype, hipStream_t st
   QRT_CHECK(a.value_dim > 0 && a.value_dim <= MAX_D, "attention: value size %d is above %d", a.value_dim, MAX_D);
   QRT_CHECK(a.chunk >= 0 && !(a.chunk > 0 && a.window > 0), "attention: a window or a chunk size, not both");
   QRT_CHECK(a.softcap >= 0.f, "attention: negative score cap");
+  QRT_CHECK(a.keep_first >= 0 && (a.keep_first == 0 || a.window > 0), "attention: first keys are kept beside a window");
   QRT_CHECK(a.nq <= 65535, "attention: too many heads");
   if (a.num_tokens == 0) return 0;
   dim3 grid(a.num_tokens, a.nq), block(64);

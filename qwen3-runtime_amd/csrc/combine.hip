@@ -158,3 +158,118 @@ extern "C" int qrt_gated_act(const void* gu, void* out, int dtype, int num_token
   QRT_LAUNCH_CHECK("gated_act");
   return 0;
 }
+
+// ------------------------------------------------ a sub-layer output with a norm of its own
+// r = rows ? rows[b] : b
+// d = y[r] / rms(y[r]) * w_after;  x = residual[r] + d  (written back without `rows`);
+// out[b] = x / rms(x) * w.  Both rms with their eps inside the root, everything float32.
+// One block of 1,024 threads per row; a thread keeps its elements in registers (rows up to 4,096
+// wide; the rest of a wider row is read again), all of them and the weights asked for first.
+template <typename TO>
+__global__ __launch_bounds__(1024) void norm_add_rmsnorm_kernel(float* __restrict__ residual, Planes y,
+                                                                const float* __restrict__ w_after, float eps_after,
+                                                                const float* __restrict__ weight, float eps,
+                                                                const int* __restrict__ rows, TO* __restrict__ out, int hidden) {
+  __shared__ float red[32];
+  const int b = blockIdx.x;
+  const int r = rows ? rows[b] : b;
+  const size_t row = (size_t)r * hidden;
+  float vy[NM_KEEP], vx[NM_KEEP], wa[NM_KEEP], wn[NM_KEEP];
+#pragma unroll
+  for (int j = 0; j < NM_KEEP; ++j) {
+    const int i = min((int)threadIdx.x + 1024 * j, hidden - 1);
+    vy[j] = planes_at(y, row + i);
+    vx[j] = residual[row + i];
+    wa[j] = w_after[i];
+    wn[j] = weight[i];
+  }
+  float sy = 0.f;
+#pragma unroll
+  for (int j = 0; j < NM_KEEP; ++j)
+    if ((int)threadIdx.x + 1024 * j < hidden) sy += vy[j] * vy[j];
+  for (int i = threadIdx.x + 1024 * NM_KEEP; i < hidden; i += 1024) {
+    const float v = planes_at(y, row + i);
+    sy += v * v;
+  }
+  sy = block_sum(sy, red);
+  const float iy = 1.0f / sqrtf(sy / (float)hidden + eps_after);
+  float sx = 0.f;
+#pragma unroll
+  for (int j = 0; j < NM_KEEP; ++j) {
+    const int i = threadIdx.x + 1024 * j;
+    if (i < hidden) {
+      vx[j] += vy[j] * iy * wa[j];
+      sx += vx[j] * vx[j];
+      if (!rows) residual[row + i] = vx[j];
+    }
+  }
+  for (int i = threadIdx.x + 1024 * NM_KEEP; i < hidden; i += 1024) {
+    const float x = residual[row + i] + planes_at(y, row + i) * iy * w_after[i];
+    sx += x * x;
+    if (!rows) residual[row + i] = x;
+  }
+  sx = block_sum(sx, red);
+  const float ix = 1.0f / sqrtf(sx / (float)hidden + eps);
+#pragma unroll
+  for (int j = 0; j < NM_KEEP; ++j) {
+    const int i = threadIdx.x + 1024 * j;
+    if (i < hidden) out[(size_t)b * hidden + i] = from_f32<TO>(vx[j] * ix * wn[j]);
+  }
+  for (int i = threadIdx.x + 1024 * NM_KEEP; i < hidden; i += 1024) {
+    const float x = rows ? residual[row + i] + planes_at(y, row + i) * iy * w_after[i] : residual[row + i];
+    out[(size_t)b * hidden + i] = from_f32<TO>(x * ix * weight[i]);
+  }
+}
+
+extern "C" int qrt_norm_add_rmsnorm(float* residual, const void* y, int y_code, int y_planes, long plane_stride,
+                                    const float* w_after, float eps_after, const float* weight, float eps, const int* rows,
+                                    void* out, int out_dtype, int num_out, int hidden, hipStream_t stream) {
+  QRT_CHECK(num_out >= 0 && hidden > 0 && y_planes >= 1, "norm_add_rmsnorm: bad sizes");
+  QRT_CHECK(y_code == QRT_F32 || (y_code == QRT_BF16 && y_planes == 1), "norm_add_rmsnorm: planes are float32");
+  if (num_out == 0) return 0;
+  const Planes yp{y, y_code, y_planes, plane_stride};
+  if (out_dtype == QRT_F32)
+    norm_add_rmsnorm_kernel<float><<<num_out, 1024, 0, stream>>>(residual, yp, w_after, eps_after, weight, eps, rows, (float*)out, hidden);
+  else if (out_dtype == QRT_BF16)
+    norm_add_rmsnorm_kernel<bf16_t><<<num_out, 1024, 0, stream>>>(residual, yp, w_after, eps_after, weight, eps, rows, (bf16_t*)out, hidden);
+  else return qrt_fail("norm_add_rmsnorm: unknown dtype %d", out_dtype);
+  QRT_LAUNCH_CHECK("norm_add_rmsnorm");
+  return 0;
+}
+
+// ------------------------------------------------ small elementwise steps
+// x *= factor, float32, in place (logits times a constant)
+__global__ void scale_kernel(float* __restrict__ x, float factor, long n) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] *= factor;
+}
+
+extern "C" int qrt_scale(float* x, float factor, long n, hipStream_t stream) {
+  QRT_CHECK(n >= 0, "scale: bad size");
+  if (n == 0) return 0;
+  scale_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0, stream>>>(x, factor, n);
+  QRT_LAUNCH_CHECK("scale");
+  return 0;
+}
+
+// activations without a gate, float32 inside. RELU2: max(x, 0)^2.
+#define QRT_UNARY_RELU2 0
+template <typename T>
+__global__ void unary_act_kernel(const T* __restrict__ x, T* __restrict__ out, long n, int kind) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) {
+    const float v = fmaxf(to_f32<T>(x[i]), 0.f);
+    out[i] = from_f32<T>(v * v);
+  }
+}
+
+extern "C" int qrt_unary_act(const void* x, void* out, int dtype, long n, int kind, hipStream_t stream) {
+  QRT_CHECK(n >= 0 && kind == QRT_UNARY_RELU2, "unary_act: unknown activation %d", kind);
+  if (n == 0) return 0;
+  const dim3 grid((unsigned)((n + 255) / 256));
+  if (dtype == QRT_F32) unary_act_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, (float*)out, n, kind);
+  else if (dtype == QRT_BF16) unary_act_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, n, kind);
+  else return qrt_fail("unary_act: unknown dtype %d", dtype);
+  QRT_LAUNCH_CHECK("unary_act");
+  return 0;
+}

@@ -6,25 +6,25 @@
 #include <math.h>
 
 // ---------------------------------------------------------------- embedding
-// residual[t, :] = float(table[ids[t], :])            (no scaling of embeddings)
+// residual[t, :] = float(table[ids[t], :]) * scale     (scale 1: the rows as they are)
 template <typename TW>
 __global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
-                             float* __restrict__ out, int hidden) {
+                             float* __restrict__ out, int hidden, float scale) {
   const int t = blockIdx.x;
   const TW* row = table + (size_t)ids[t] * hidden;
   float* o = out + (size_t)t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_f32<TW>(row[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_f32<TW>(row[i]) * scale;
 }
 
 extern "C" int qrt_embed(const int* ids, const void* table, int table_dtype, float* out,
-                         int num_tokens, int vocab, int hidden, hipStream_t stream) {
+                         int num_tokens, int vocab, int hidden, float scale, hipStream_t stream) {
   QRT_CHECK(num_tokens >= 0 && vocab > 0 && hidden > 0, "embed: bad sizes T=%d V=%d H=%d", num_tokens, vocab, hidden);
   if (num_tokens == 0) return 0;
   dim3 grid(num_tokens), block(256);
   if (table_dtype == QRT_F32)
-    embed_kernel<float><<<grid, block, 0, stream>>>(ids, (const float*)table, out, hidden);
+    embed_kernel<float><<<grid, block, 0, stream>>>(ids, (const float*)table, out, hidden, scale);
   else if (table_dtype == QRT_BF16)
-    embed_kernel<bf16_t><<<grid, block, 0, stream>>>(ids, (const bf16_t*)table, out, hidden);
+    embed_kernel<bf16_t><<<grid, block, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, scale);
   else
     return qrt_fail("embed: unknown table dtype %d", table_dtype);
   QRT_LAUNCH_CHECK("embed");

@@ -1,0 +1,203 @@
+// Steps of attention through a latent, each over packed tokens:
+//
+// * the RMS norm of some columns of a wider matrix (a latent that a fused product left beside
+//   other things), float32 inside, out in the matrix's type;
+// * the write of the cached row: columns [first, first + rank) RMS-normed are the latent c, the
+//   rot_dim columns behind them, rotated, the key part all heads share; the key row of the one
+//   key/value head is [c | k_rot], its value row [c | 0] (keys [page, 1, offset, W], values
+//   [page, 1, W, offset], W = rank + rot_dim);
+// * a copy of `width` elements per (token, head) from one strided layout to another with the
+//   first 2 n of them turned, element i against element i + n, by position * freq[i] (the
+//   "rotate half" layout; angles, sines and cosines float32);
+// * a product per head, out[t, h, :] = W[h] x[t, h, :], on strided rows: W [heads, N, K].
+#include "common.h"
+#include <math.h>
+
+// ---------------------------------------------------------------- norm of some columns
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_columns_kernel(const T* __restrict__ y, long stride, int first, int width,
+                                                              const float* __restrict__ weight, float eps,
+                                                              T* __restrict__ out) {
+  __shared__ float red[32];
+  const T* row = y + (size_t)blockIdx.x * stride + first;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float v = to_f32<T>(row[i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += 256)
+    out[(size_t)blockIdx.x * width + i] = from_f32<T>(to_f32<T>(row[i]) * inv * weight[i]);
+}
+
+extern "C" int qrt_rmsnorm_columns(const void* y, long stride, int first, int width, const float* weight, float eps,
+                                   void* out, int dtype, int num_tokens, hipStream_t stream) {
+  QRT_CHECK(num_tokens >= 0 && width > 0 && first >= 0 && (long)first + width <= stride, "rmsnorm_columns: bad sizes");
+  if (num_tokens == 0) return 0;
+  if (dtype == QRT_F32)
+    rmsnorm_columns_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)y, stride, first, width, weight, eps, (float*)out);
+  else if (dtype == QRT_BF16)
+    rmsnorm_columns_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)y, stride, first, width, weight, eps, (bf16_t*)out);
+  else return qrt_fail("rmsnorm_columns: unknown dtype %d", dtype);
+  QRT_LAUNCH_CHECK("rmsnorm_columns");
+  return 0;
+}
+
+// ---------------------------------------------------------------- the cached row
+template <typename T>
+__global__ __launch_bounds__(256) void latent_store_kernel(const T* __restrict__ y, long stride, int first, int rank,
+                                                           int rot_dim, const float* __restrict__ weight, float eps,
+                                                           const int* __restrict__ positions, const float* __restrict__ freq,
+                                                           int pairs, const int* __restrict__ slots, T* __restrict__ k_cache,
+                                                           T* __restrict__ v_cache, int page_size) {
+  __shared__ float red[32];
+  const int t = blockIdx.x;
+  const T* row = y + (size_t)t * stride + first;
+  const int slot = slots[t];
+  const int page = slot / page_size, off = slot - page * page_size;
+  const int w = rank + rot_dim;
+  T* kr = k_cache + (size_t)slot * w;
+  T* vr = v_cache + (size_t)page * w * page_size + off;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < rank; i += 256) {
+    const float v = to_f32<T>(row[i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)rank + eps);
+  for (int i = threadIdx.x; i < rank; i += 256) {
+    const T c = from_f32<T>(to_f32<T>(row[i]) * inv * weight[i]);
+    kr[i] = c;
+    vr[(size_t)i * page_size] = c;
+  }
+  const float pos = (float)positions[t];
+  const T* rot = row + rank;
+  for (int i = threadIdx.x; i < rot_dim; i += 256) {
+    float x = to_f32<T>(rot[i]);
+    if (i < 2 * pairs) {
+      const int j = i < pairs ? i : i - pairs;
+      float sn, cs;
+      sincos_angle(pos * freq[j], &sn, &cs);
+      const float other = to_f32<T>(rot[i < pairs ? i + pairs : i - pairs]);
+      x = i < pairs ? x * cs - other * sn : x * cs + other * sn;
+    }
+    kr[rank + i] = from_f32<T>(x);
+    vr[(size_t)(rank + i) * page_size] = from_f32<T>(0.f);
+  }
+}
+
+extern "C" int qrt_latent_store(const void* y, long stride, int first, int rank, int rot_dim, const float* weight, float eps,
+                                const int* positions, const float* freq, int pairs, const int* slots, void* k_cache,
+                                void* v_cache, int page_size, long num_pages, int dtype, int num_tokens, hipStream_t stream) {
+  QRT_CHECK(num_tokens >= 0 && rank > 0 && rot_dim >= 0 && first >= 0 && (long)first + rank + rot_dim <= stride,
+            "latent_store: bad sizes");
+  QRT_CHECK(pairs >= 0 && 2 * pairs <= rot_dim && (pairs == 0 || freq), "latent_store: %d pairs in %d elements", pairs, rot_dim);
+  QRT_CHECK(page_size > 0 && num_pages > 0 && slots && positions, "latent_store: no cache");
+  if (num_tokens == 0) return 0;
+  if (dtype == QRT_F32)
+    latent_store_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)y, stride, first, rank, rot_dim, weight, eps, positions,
+                                                               freq, pairs, slots, (float*)k_cache, (float*)v_cache, page_size);
+  else if (dtype == QRT_BF16)
+    latent_store_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)y, stride, first, rank, rot_dim, weight, eps, positions,
+                                                                freq, pairs, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size);
+  else return qrt_fail("latent_store: unknown dtype %d", dtype);
+  QRT_LAUNCH_CHECK("latent_store");
+  return 0;
+}
+
+// ---------------------------------------------------------------- rotate half, from one layout to another
+struct RotateArgs {
+  const void* x; long x_row; int in_stride, in_offset;
+  void* out; long out_row; int out_stride, out_offset;
+  int heads, width, pairs;
+  const int* positions; const float* freq;
+  int scale_from_head; float scale;  // heads from this one on are multiplied by `scale` after turning
+};
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void rotate_half_kernel(RotateArgs a) {
+  const int t = blockIdx.x;
+  const float pos = a.pairs ? (float)a.positions[t] : 0.f;
+  const TI* xr = (const TI*)a.x + (size_t)t * a.x_row + a.in_offset;
+  TO* orow = (TO*)a.out + (size_t)t * a.out_row + a.out_offset;
+  const int total = a.heads * a.width;
+  for (int e = blockIdx.y * 256 + threadIdx.x; e < total; e += 256 * gridDim.y) {
+    const int h = e / a.width, i = e - h * a.width;
+    const TI* src = xr + (size_t)h * a.in_stride;
+    float x = to_f32<TI>(src[i]);
+    if (i < 2 * a.pairs) {
+      const int j = i < a.pairs ? i : i - a.pairs;
+      float sn, cs;
+      sincos_angle(pos * a.freq[j], &sn, &cs);
+      const float other = to_f32<TI>(src[i < a.pairs ? i + a.pairs : i - a.pairs]);
+      x = i < a.pairs ? x * cs - other * sn : x * cs + other * sn;
+    }
+    if (h >= a.scale_from_head) x *= a.scale;
+    orow[(size_t)h * a.out_stride + i] = from_f32<TO>(x);
+  }
+}
+
+extern "C" int qrt_rotate_half(const RotateArgs* args, int in_dtype, int out_dtype, int num_tokens, hipStream_t stream) {
+  RotateArgs a = *args;
+  QRT_CHECK(num_tokens >= 0 && a.heads > 0 && a.width > 0 && a.pairs >= 0 && 2 * a.pairs <= a.width, "rotate_half: bad sizes");
+  QRT_CHECK(a.in_offset >= 0 && a.in_offset + a.width <= a.in_stride && (long)a.heads * a.in_stride <= a.x_row &&
+            a.out_offset >= 0 && a.out_offset + a.width <= a.out_stride && (long)a.heads * a.out_stride <= a.out_row,
+            "rotate_half: heads of %d at %d in rows of %ld, to heads of %d at %d in rows of %ld", a.in_stride, a.in_offset,
+            a.x_row, a.out_stride, a.out_offset, a.out_row);
+  QRT_CHECK(a.pairs == 0 || (a.freq && a.positions), "rotate_half: no angles");
+  if (num_tokens == 0) return 0;
+  const int total = a.heads * a.width;
+  const dim3 grid(num_tokens, num_tokens >= 512 ? 1 : min((total + 255) / 256, 64));
+  if (in_dtype == QRT_F32 && out_dtype == QRT_F32) rotate_half_kernel<float, float><<<grid, 256, 0, stream>>>(a);
+  else if (in_dtype == QRT_BF16 && out_dtype == QRT_BF16) rotate_half_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>(a);
+  else if (in_dtype == QRT_BF16 && out_dtype == QRT_F32) rotate_half_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(a);
+  else return qrt_fail("rotate_half: no form for types %d -> %d", in_dtype, out_dtype);
+  QRT_LAUNCH_CHECK("rotate_half");
+  return 0;
+}
+
+// ---------------------------------------------------------------- a product per head
+// One block of four waves per (token, head): the head's input in LDS as float32, each wave takes
+// outputs wave, wave + 4, ...; an output is one wave's sum over K in a fixed order, whatever else is
+// in the batch. For few tokens and for float32; many tokens in bfloat16 go to a batched library product.
+template <typename T>
+__global__ __launch_bounds__(256) void heads_linear_kernel(const T* __restrict__ x, long x_row, int in_stride, int in_offset,
+                                                           const T* __restrict__ w, int n, int k, T* __restrict__ out,
+                                                           long out_row, int out_stride, int out_offset) {
+  extern __shared__ float xs[];
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* xr = x + (size_t)t * x_row + (size_t)h * in_stride + in_offset;
+  for (int i = threadIdx.x; i < k; i += 256) xs[i] = to_f32<T>(xr[i]);
+  __syncthreads();
+  const T* wh = w + (size_t)h * n * k;
+  T* o = out + (size_t)t * out_row + (size_t)h * out_stride + out_offset;
+  for (int j = wave; j < n; j += 4) {
+    const T* wr = wh + (size_t)j * k;
+    float acc = 0.f;
+    for (int c = lane; c < k; c += 64) acc = fmaf(xs[c], to_f32<T>(wr[c]), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) o[j] = from_f32<T>(acc);
+  }
+}
+
+extern "C" int qrt_heads_linear(const void* x, long x_row, int in_stride, int in_offset, const void* w, int heads, int n, int k,
+                                void* out, long out_row, int out_stride, int out_offset, int dtype, int num_tokens,
+                                hipStream_t stream) {
+  QRT_CHECK(num_tokens >= 0 && heads > 0 && heads <= 65535 && n > 0 && k > 0 && k <= 16384, "heads_linear: bad sizes");
+  QRT_CHECK(in_offset >= 0 && in_offset + k <= in_stride && (long)heads * in_stride <= x_row && out_offset >= 0 &&
+            out_offset + n <= out_stride && (long)heads * out_stride <= out_row, "heads_linear: heads do not fit their rows");
+  if (num_tokens == 0) return 0;
+  const dim3 grid(num_tokens, heads);
+  const size_t lds = (size_t)k * sizeof(float);
+  if (dtype == QRT_F32)
+    heads_linear_kernel<float><<<grid, 256, lds, stream>>>((const float*)x, x_row, in_stride, in_offset, (const float*)w, n, k,
+                                                           (float*)out, out_row, out_stride, out_offset);
+  else if (dtype == QRT_BF16)
+    heads_linear_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, x_row, in_stride, in_offset, (const bf16_t*)w, n, k,
+                                                            (bf16_t*)out, out_row, out_stride, out_offset);
+  else return qrt_fail("heads_linear: unknown dtype %d", dtype);
+  QRT_LAUNCH_CHECK("heads_linear");
+  return 0;
+}

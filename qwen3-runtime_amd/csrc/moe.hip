@@ -3,9 +3,10 @@
 //
 // Router: logits z[e] = x . W_r[e] + b[e] in float32 (the router's matrix is held in float32
 // in every mode), the `top` largest per token (ties: the lower index), softmax over those; or,
-// with sigmoid scores, the `top` largest sigmoid(z), which weigh the experts as they are. Experts
+// with sigmoid scores, the `top` largest sigmoid(z), which weigh the experts as they are; or, with
+// softmax scores over all experts (`sigmoid_scores` = 2), the `top` largest of those, likewise. Experts
 // may form equal groups of neighbours of which only the `keep` best (by the sum of a group's two
-// largest entries) stay in the choice.
+// largest entries, or with `group_max` by its largest) stay in the choice.
 // Experts: pair p = (token t, its j-th expert e) computes act[p] = silu(G_e x) * (U_e x) (or the
 // clamped activation of common.h) with
 // gate_up [E, 2I, H] (gate rows, then up rows), then out[t] = sum_j w[t, j] * D_e act[p] with
@@ -43,7 +44,7 @@ template <typename T>
 __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x, const float* __restrict__ router,
                                                          const float* __restrict__ bias, int* __restrict__ index,
                                                          float* __restrict__ weight, int hidden, int experts, int top,
-                                                         int sigmoid_scores, int groups, int keep) {
+                                                         int sigmoid_scores, int groups, int keep, int group_max) {
   __shared__ float logit[MAX_EXPERTS];
   __shared__ float score[MAX_EXPERTS];
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -69,9 +70,17 @@ __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x
   }
   __syncthreads();
   if (wave != 0) return;
-  if (sigmoid_scores) {
+  if (sigmoid_scores == 1) {
     // scores sigmoid(z) take the logits' place: the choice goes by them, and they are the weights
     for (int e = lane; e < experts; e += 64) score[e] = logit[e] = 1.0f / (1.0f + expf(-logit[e]));
+    __builtin_amdgcn_wave_barrier();
+  } else if (sigmoid_scores == 2) {
+    // the softmax over all experts likewise; maximum and sum in the same order in every lane
+    float mx = -INFINITY, sum = 0.f;
+    for (int e = 0; e < experts; ++e) mx = fmaxf(mx, logit[e]);
+    for (int e = 0; e < experts; ++e) sum += expf(logit[e] - mx);
+    __builtin_amdgcn_wave_barrier();
+    for (int e = lane; e < experts; e += 64) score[e] = logit[e] = expf(logit[e] - mx) / sum;
     __builtin_amdgcn_wave_barrier();
   }
   if (groups > 1 && keep < groups) {
@@ -85,7 +94,7 @@ __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x
         const float z = logit[e];
         if (z > a) { b = a; a = z; } else if (z > b) b = z;
       }
-      mine = per > 1 ? a + b : a;
+      mine = (per > 1 && !group_max) ? a + b : a;
     }
     bool kept = false;
     for (int j = 0; j < keep; ++j) {
@@ -135,7 +144,7 @@ __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x
 
 extern "C" int qrt_route_top(const void* x, int x_dtype, const float* router, const float* bias, int* index,
                              float* weight, int num_tokens, int hidden, int experts, int top, int sigmoid_scores,
-                             int groups, int keep, hipStream_t stream) {
+                             int groups, int keep, int group_max, hipStream_t stream) {
   QRT_CHECK(groups >= 1 && groups <= 64 && experts % groups == 0 && keep >= 1 && keep <= groups &&
             (long)keep * (experts / groups) >= top,
             "route_top: %d groups of which %d stay do not fit %d experts of which %d are chosen", groups, keep, experts, top);
@@ -145,9 +154,9 @@ extern "C" int qrt_route_top(const void* x, int x_dtype, const float* router, co
   if (num_tokens == 0) return 0;
   dim3 grid(num_tokens), block(1024);
   if (x_dtype == QRT_F32)
-    route_top_kernel<float><<<grid, block, 0, stream>>>((const float*)x, router, bias, index, weight, hidden, experts, top, sigmoid_scores, groups, keep);
+    route_top_kernel<float><<<grid, block, 0, stream>>>((const float*)x, router, bias, index, weight, hidden, experts, top, sigmoid_scores, groups, keep, group_max);
   else if (x_dtype == QRT_BF16)
-    route_top_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, router, bias, index, weight, hidden, experts, top, sigmoid_scores, groups, keep);
+    route_top_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, router, bias, index, weight, hidden, experts, top, sigmoid_scores, groups, keep, group_max);
   else return qrt_fail("route_top: unknown dtype %d", x_dtype);
   QRT_LAUNCH_CHECK("route_top");
   return 0;

@@ -134,7 +134,7 @@ class ModelRunner:
 
     def _context(self, packed: PackedStep, dev: dict[str, torch.Tensor]) -> StepContext:
         groups = [
-            GroupView(g.page_size, g.window, dev[f"table{gi}"], dev[f"slots{gi}"], g.chunk)
+            GroupView(g.page_size, g.window, dev[f"table{gi}"], dev[f"slots{gi}"], g.chunk, g.keep_first)
             for gi, g in enumerate(self.cache.groups)
         ]
         return StepContext(

@@ -55,6 +55,7 @@ class _AttnArgs(Structure):
         ("table_width", c_int), ("num_tokens", c_int), ("nq", c_int), ("nkv", c_int),
         ("head_dim", c_int), ("page_size", c_int), ("window", c_int), ("scale", c_float),
         ("chunk", c_int), ("softcap", c_float), ("value_dim", c_int), ("gate", c_void_p), ("gate_stride", c_long),
+        ("keep_first", c_int), ("sink", c_int),
     ]
 
 
@@ -91,6 +92,23 @@ class _ConvArgs(Structure):
         ("num_tokens", c_int), ("channels", c_int), ("num_taps", c_int), ("nseg", c_int),
         ("seg_first", c_int * 4), ("seg_heads", c_int * 4), ("seg_width", c_int * 4), ("seg_mode", c_int * 4),
         ("total_heads", c_int), ("unit_eps", c_float), ("fuse_tail", c_int),
+    ]
+
+
+class _RotateArgs(Structure):
+    _fields_ = [
+        ("x", c_void_p), ("x_row", c_long), ("in_stride", c_int), ("in_offset", c_int),
+        ("out", c_void_p), ("out_row", c_long), ("out_stride", c_int), ("out_offset", c_int),
+        ("heads", c_int), ("width", c_int), ("pairs", c_int),
+        ("positions", c_void_p), ("freq", c_void_p), ("scale_from_head", c_int), ("scale", c_float),
+    ]
+
+
+class _RetentionArgs(Structure):
+    _fields_ = [
+        ("qkv", c_void_p), ("channels", c_int), ("q_first", c_int), ("k_first", c_int), ("v_first", c_int),
+        ("decay", c_void_p), ("state", c_void_p), ("out", c_void_p), ("cu_q", c_void_p), ("state_slots", c_void_p),
+        ("heads", c_int), ("dim", c_int), ("vdim", c_int),
     ]
 
 
@@ -238,16 +256,38 @@ class HipOps:
             raise OpsError(lib.qrt_last_error().decode())
 
     # ---- embedding, norms, activations ---------------------------------------
-    def embed(self, ids, table):
+    def embed(self, ids, table, scale=1.0):
         _need(ids, "ids", torch.int32)
         _need(table, "embedding table")
         t, (v, h) = ids.numel(), table.shape
         out = torch.empty((t, h), dtype=torch.float32, device=table.device)
         self._check(self.lib, self.lib.qrt_embed(_ptr(ids), _ptr(table), _CODE[table.dtype], _ptr(out),
-                                                 c_int(t), c_int(v), c_int(h), _stream()))
+                                                 c_int(t), c_int(v), c_int(h), c_float(scale), _stream()))
         return out
 
-    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None, delta_scale=1.0):
+    def scale(self, x, factor):
+        """``x *= factor`` in place, float32."""
+        _need(x, "x", torch.float32)
+        self._check(self.lib, self.lib.qrt_scale(_ptr(x), c_float(factor), c_long(x.numel()), _stream()))
+        return x
+
+    def unary_act(self, x, kind):
+        """An activation without a gate, element by element: ``relu2`` is ``max(x, 0)^2``."""
+        _need(x, "x")
+        out = torch.empty_like(x)
+        self._check(self.lib, self.lib.qrt_unary_act(_ptr(x), _ptr(out), _CODE[x.dtype], c_long(x.numel()),
+                                                     c_int({"relu2": 0}[kind]), _stream()))
+        return out
+
+    def new_rows(self, t, width, dtype, device):
+        return torch.empty((t, width), dtype=dtype, device=device)
+
+    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None, delta_scale=1.0, delta_norm=None):
+        """``residual += delta_scale * delta`` in place (``delta`` a matrix or float32 planes), then the
+        rows' RMS norm; with ``rows`` only those, and ``residual`` is left alone. ``delta_norm`` =
+        (weight, eps): ``delta`` joins the stream as ``delta / rms(delta) * weight``."""
+        if delta_norm is not None:
+            return self._norm_add_rmsnorm(residual, delta, delta_norm[0], delta_norm[1], weight, eps, out_dtype, rows)
         t, h = residual.shape
         _need(residual, "residual", torch.float32)
         _need(weight, "norm weight", torch.float32, (h,))
@@ -267,6 +307,143 @@ class HipOps:
             _ptr(residual), _ptr(delta), _CODE[delta.dtype] if delta is not None else F32, _ptr(weight),
             _ptr(rows), _ptr(out), _CODE[out_dtype], c_int(n_out), c_int(h), c_float(eps), c_int(planes),
             c_long(plane_stride), c_float(delta_scale), _stream()))
+        return out
+
+    def _norm_add_rmsnorm(self, residual, y, w_after, eps_after, weight, eps, out_dtype, rows):
+        t, h = residual.shape
+        _need(residual, "residual", torch.float32)
+        _need(weight, "norm weight", torch.float32, (h,))
+        _need(w_after, "weight of the norm behind the sub-layer", torch.float32, (h,))
+        py, cy, ny = _planes(y, t, h, "sub-layer output")
+        n_out = t
+        if rows is not None:
+            _need(rows, "rows", torch.int32)
+            n_out = rows.numel()
+        out = torch.empty((n_out, h), dtype=out_dtype, device=residual.device)
+        self._check(self.lib, self.lib.qrt_norm_add_rmsnorm(
+            _ptr(residual), py, c_int(cy), c_int(ny), c_long(t * h), _ptr(w_after), c_float(eps_after), _ptr(weight),
+            c_float(eps), _ptr(rows), _ptr(out), _CODE[out_dtype], c_int(n_out), c_int(h), _stream()))
+        return out
+
+    # ---- attention through a latent, retention ------------------------------------------
+    def rmsnorm_columns(self, y, first, width, weight, eps):
+        """The RMS norm of columns ``first .. first + width`` of ``y`` [T, W], [T, width] in ``y``'s type."""
+        t, w = y.shape
+        _need(y, "y")
+        _need(weight, "norm weight", torch.float32, (width,))
+        if not 0 <= first <= first + width <= w:
+            raise OpsError(f"columns {first}..{first + width} of {w}")
+        out = torch.empty((t, width), dtype=y.dtype, device=y.device)
+        self._check(self.lib, self.lib.qrt_rmsnorm_columns(_ptr(y), c_long(w), c_int(first), c_int(width), _ptr(weight),
+                                                           c_float(eps), _ptr(out), _CODE[y.dtype], c_int(t), _stream()))
+        return out
+
+    def latent_store(self, y, first, rank, rot_dim, weight, eps, positions, freq, cache):
+        """Columns ``first .. first + rank`` of ``y`` RMS-normed (the latent ``c``) and the ``rot_dim``
+        columns behind them rotated (rotate-half over the first ``2 len(freq)``) go into the cache of
+        one key/value head: the key row ``[c | k_rot]``, the value row ``[c | 0]``."""
+        if cache is None:
+            return
+        t, w = y.shape
+        width = rank + rot_dim
+        _need(y, "y")
+        _need(weight, "latent norm weight", torch.float32, (rank,))
+        pairs = 0 if freq is None else freq.numel()
+        if pairs:
+            _need(freq, "freq", torch.float32, (pairs,))
+        _need(positions, "positions", torch.int32, (t,))
+        pages = self._check_cache(cache, 1, width, y.dtype)
+        _need(cache.group.slots, "slots", torch.int32, (t,))
+        if not 0 <= first <= first + width <= w or 2 * pairs > rot_dim:
+            raise OpsError(f"latent_store: columns {first}..{first + width} of {w}, {pairs} pairs in {rot_dim}")
+        self._check(self.lib, self.lib.qrt_latent_store(
+            _ptr(y), c_long(w), c_int(first), c_int(rank), c_int(rot_dim), _ptr(weight), c_float(eps), _ptr(positions),
+            _ptr(freq), c_int(pairs), _ptr(cache.group.slots), _ptr(cache.k), _ptr(cache.v), c_int(cache.group.page_size),
+            c_long(pages), _CODE[y.dtype], c_int(t), _stream()))
+
+    def rotate_half(self, x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq,
+                    scale_from_head=None, scale=1.0):
+        """For every token and head copy ``width`` elements from ``x[t, h * in_stride + in_offset ...]`` to
+        ``out[t, h * out_stride + out_offset ...]``, the first ``2 len(freq)`` of them turned (element i
+        against element i + len(freq), by ``position * freq[i]``); heads from ``scale_from_head`` on are
+        multiplied by ``scale``. ``out`` may be float32 for a bfloat16 ``x``."""
+        t = x.shape[0]
+        _need(x, "x")
+        _need(out, "out", shape=(t, out.shape[1]))
+        pairs = 0 if freq is None else freq.numel()
+        a = _RotateArgs()
+        a.x, a.x_row, a.in_stride, a.in_offset = x.data_ptr(), x.shape[1], in_stride, in_offset
+        a.out, a.out_row, a.out_stride, a.out_offset = out.data_ptr(), out.shape[1], out_stride, out_offset
+        a.heads, a.width, a.pairs = heads, width, pairs
+        if pairs:
+            a.freq = _need(freq, "freq", torch.float32, (pairs,)).data_ptr()
+            a.positions = _need(positions, "positions", torch.int32, (t,)).data_ptr()
+        a.scale_from_head, a.scale = heads if scale_from_head is None else scale_from_head, scale
+        self._check(self.lib, self.lib.qrt_rotate_half(byref(a), _CODE[x.dtype], _CODE[out.dtype], c_int(t), _stream()))
+        return out
+
+    # bfloat16 steps with more tokens than this take the per-head products to the vendor library
+    heads_linear_own_max_rows = 16
+
+    def heads_linear(self, x, in_stride, in_offset, w, out, out_stride, out_offset):
+        """A product per head on strided rows: ``out[t, h * out_stride + out_offset + n] =
+        sum_k w[h, n, k] x[t, h * in_stride + in_offset + k]``; ``w`` [heads, N, K]."""
+        t = x.shape[0]
+        heads, n, k = w.shape
+        _need(x, "x")
+        _need(w, "weights", x.dtype)
+        _need(out, "out", x.dtype, (t, out.shape[1]))
+        if (heads * in_stride > x.shape[1] or in_offset + k > in_stride or heads * out_stride > out.shape[1]
+                or out_offset + n > out_stride):
+            raise OpsError(f"heads_linear: {heads} heads of {in_stride} in rows of {x.shape[1]}, of {out_stride} in rows of {out.shape[1]}")
+        if x.dtype == torch.bfloat16 and t > self.heads_linear_own_max_rows:
+            src = x.view(t, -1)[:, : heads * in_stride].view(t, heads, in_stride)[:, :, in_offset: in_offset + k]
+            res = torch.bmm(src.transpose(0, 1), w.transpose(1, 2))  # [heads, T, N]
+            out.view(t, -1)[:, : heads * out_stride].view(t, heads, out_stride)[:, :, out_offset: out_offset + n] = \
+                res.transpose(0, 1)
+            return out
+        self._check(self.lib, self.lib.qrt_heads_linear(
+            _ptr(x), c_long(x.shape[1]), c_int(in_stride), c_int(in_offset), _ptr(w), c_int(heads), c_int(n), c_int(k),
+            _ptr(out), c_long(out.shape[1]), c_int(out_stride), c_int(out_offset), _CODE[x.dtype], c_int(t), _stream()))
+        return out
+
+    def retention_prepare(self, y, heads, dim, vdim, positions, freq, k_scale):
+        """float32 [T, 2 heads dim + heads vdim] from the first columns of a product ``y``: queries and
+        keys with their first ``2 len(freq)`` elements a head turned (rotate-half), keys then times
+        ``k_scale``, values as they are."""
+        t, w = y.shape
+        c = 2 * heads * dim + heads * vdim
+        if c > w:
+            raise OpsError(f"retention_prepare: {c} channels in {w} columns")
+        out = torch.empty((t, c), dtype=torch.float32, device=y.device)
+        self.rotate_half(y, dim, 0, out, dim, 0, 2 * heads, dim, positions, freq, scale_from_head=heads, scale=k_scale)
+        # the values: a copy into float32 behind them
+        a = _RotateArgs()
+        _need(y, "y")
+        a.x, a.x_row, a.in_stride, a.in_offset = y.data_ptr() + 2 * heads * dim * y.element_size(), w, vdim, 0
+        a.out, a.out_row, a.out_stride, a.out_offset = out.data_ptr() + 2 * heads * dim * 4, c, vdim, 0
+        a.heads, a.width, a.pairs, a.scale_from_head, a.scale = heads, vdim, 0, heads, 1.0
+        self._check(self.lib, self.lib.qrt_rotate_half(byref(a), _CODE[y.dtype], F32, c_int(t), _stream()))
+        return out
+
+    def retention_rule(self, ctx, qkv, decay, state, heads, dim, vdim):
+        """``S <- decay S + k v^T; o = S^T q`` over each sequence's tokens from its slot's state (float32
+        [slots, heads, vdim, dim], updated in place); ``qkv`` float32 [T, C] as ``retention_prepare``
+        leaves it. Returns the read-outs, float32 [T, heads, vdim]."""
+        t = ctx.num_tokens
+        c = 2 * heads * dim + heads * vdim
+        _need(qkv, "q | k | v", torch.float32, (t, c))
+        _need(state, "state", torch.float32, (state.shape[0], heads, vdim, dim))
+        _need(decay, "decay", torch.float32, (heads,))
+        a = _RetentionArgs()
+        a.qkv, a.channels, a.q_first, a.k_first, a.v_first = qkv.data_ptr(), c, 0, heads * dim, 2 * heads * dim
+        a.decay, a.state = decay.data_ptr(), state.data_ptr()
+        out = torch.empty((t, heads, vdim), dtype=torch.float32, device=qkv.device)
+        a.out = out.data_ptr()
+        a.cu_q = _need(ctx.cu_q, "cu_q", torch.int32, (ctx.num_seqs + 1,)).data_ptr()
+        a.state_slots = _need(ctx.state_slots, "state_slots", torch.int32, (ctx.num_seqs,)).data_ptr()
+        a.heads, a.dim, a.vdim = heads, dim, vdim
+        self._check(self.lib, self.lib.qrt_retention(byref(a), c_int(t), c_int(ctx.num_seqs), c_int(state.shape[0]), _stream()))
         return out
 
     # ---- steps between sub-layers that are neither a product nor a plain norm -----------
@@ -447,12 +624,13 @@ class HipOps:
         return out
 
     # ---- routed experts --------------------------------------------------------------
-    def route_top(self, x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None):
+    def route_top(self, x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None, group_score="top2"):
         """Router logits ``x W^T + b`` in float32, the ``top`` largest per token and the softmax
         over those alone: (int32 [T, top], float32 [T, top]). ``scoring="sigmoid"``: the choice goes
-        by ``sigmoid`` of the logits, which are also the weights, as they are. ``groups``, ``keep``:
-        only experts of the ``keep`` best of ``groups`` equal groups of neighbours can be chosen, a
-        group's score being the sum of its two largest entries."""
+        by ``sigmoid`` of the logits, which are also the weights, as they are; ``"softmax_all"``: by the
+        softmax over all experts' logits, likewise. ``groups``, ``keep``: only experts of the ``keep``
+        best of ``groups`` equal groups of neighbours can be chosen, a group's score being the sum of
+        its two largest entries (``group_score="top2"``) or its largest (``"max"``)."""
         t, h = x.shape
         _need(x, "x")
         n = router.shape[0]
@@ -463,8 +641,9 @@ class HipOps:
         weight = torch.empty((t, top), dtype=torch.float32, device=x.device)
         self._check(self.lib, self.lib.qrt_route_top(_ptr(x), _CODE[x.dtype], _ptr(router), _ptr(router_bias),
                                                      _ptr(index), _ptr(weight), c_int(t), c_int(h), c_int(n),
-                                                     c_int(top), c_int(scoring == "sigmoid"), c_int(groups),
-                                                     c_int(groups if keep is None else keep), _stream()))
+                                                     c_int(top), c_int({"softmax_top": 0, "sigmoid": 1, "softmax_all": 2}[scoring]),
+                                                     c_int(groups), c_int(groups if keep is None else keep),
+                                                     c_int(group_score == "max"), _stream()))
         return index, weight
 
     def moe_swiglu(self, x, gate_up, down, index, weight, activation="swiglu", limit=0.0, out=None):
@@ -883,12 +1062,12 @@ class HipOps:
         return table
 
     def fuses_decode_attention(self, ctx, qkv, nq, nkv, d, cache, value_dim=None, chunk=None, softcap=None,
-                               gate=None) -> bool:
+                               gate=None, keep_first=0, sink=False) -> bool:
         """Whether ``decode_attention`` serves this step: one token per sequence, bfloat16, a head
         size that keeps a rotation pair in one lane (a multiple of 64, up to 256), at most 16
         query heads per key head, and a layer that writes its own cache."""
-        if value_dim not in (None, d):
-            return False
+        if value_dim not in (None, d) or keep_first or sink:
+            return False  # the kept keys and the sink join in the merge of parts, which reads the queries
         return (self.fuse_decode and qkv.dtype == torch.bfloat16 and ctx.max_q_len == 1
                 and ctx.num_tokens == ctx.num_seqs and d % 64 == 0 and d <= 256 and nq // nkv <= 16
                 and cache is not None and cache.writes and cache.group.page_size % 8 == 0
@@ -925,7 +1104,7 @@ class HipOps:
         return out
 
     def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window, chunk=None, softcap=None, value_dim=None,
-                        gate=None):
+                        gate=None, keep_first=0, sink=False):
         """Attention of every query over its sequence's cache. Beyond the plain form: a mask of
         chunks instead of a window (``chunk``), a tanh cap on the scaled scores (``softcap``),
         values of ``value_dim`` elements, and a ``gate`` [T, nq * value_dim] (columns of a wider
@@ -944,7 +1123,9 @@ class HipOps:
         if table.shape[1] < need_pages:
             raise OpsError(f"block table is {table.shape[1]} pages wide, the longest sequence needs {need_pages}")
         out = torch.empty((t, nq * dv), dtype=q.dtype, device=q.device)
-        if dv == d and q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0:
+        if keep_first and not window:
+            raise OpsError("first keys are kept in sight beside a window")
+        if dv == d and q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0 and not keep_first and not sink:
             self._attention_mfma(q, out, cache, ctx, nq, nkv, d, scale, window or 0, chunk or 0, softcap or 0.0, gate)
         else:
             a = _AttnArgs()
@@ -957,6 +1138,7 @@ class HipOps:
             a.chunk, a.softcap, a.value_dim = chunk or 0, softcap or 0.0, dv
             if gate is not None:
                 a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
+            a.keep_first, a.sink = int(keep_first), int(bool(sink))
             self._check(self.lib, self.lib.qrt_attention_f32(byref(a), _CODE[q.dtype], _stream()))
         return out
 

@@ -1,6 +1,6 @@
 """Layer parts. Importing this package registers the shipped kinds."""
 
-from . import attention, block, delta, embedding, entry, mlp, moe, norm, parallel, rope  # noqa: F401
+from . import attention, block, delta, embedding, entry, latent, mlp, moe, norm, parallel, retention, rope  # noqa: F401
 from .base import (  # noqa: F401
     Block,
     CacheView,
@@ -8,6 +8,7 @@ from .base import (  # noqa: F401
     GroupView,
     Mixer,
     Norm,
+    NormedUpdate,
     Part,
     PositionEncoding,
     StepContext,

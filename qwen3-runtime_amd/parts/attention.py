@@ -19,7 +19,10 @@ by their root mean square); a fixed score ``scale``; a cap on the scaled scores,
 from position 0 of the sequence); an output gate (``output_gate``: one more projection ``g`` of
 the mixer's input, whose sigmoid multiplies the concatenated heads before the output projection);
 biases on the q, k and v projections (``bias``: tensors ``q_bias``, ``k_bias``, ``v_bias``, added to the
-product's output in float32, before any rotation).
+product's output in float32, before any rotation); beside a window, the sequence's first
+``keep_first`` tokens stay visible to every later query (key ``j`` is visible iff ``j <= i`` and
+``i - j < window or j < keep_first``; the cache keeps their pages); a ``sink`` in the softmax, one more
+term of score 0 and no value in its denominator (``p_j = exp(s_j) / (1 + sum exp(s_j))``).
 """
 
 from __future__ import annotations
@@ -51,6 +54,8 @@ class GroupedQueryAttention(Mixer):
         chunk: int | None = None,
         output_gate: bool = False,
         bias: bool = False,
+        keep_first: int = 0,
+        sink: bool = False,
         tensors=None,
     ):
         super().__init__(tensors)
@@ -71,6 +76,9 @@ class GroupedQueryAttention(Mixer):
         self.output_gate = bool(output_gate)
         self.has_bias = bool(bias)
         self.bias = None
+        self.keep_first, self.sink = int(keep_first), bool(sink)
+        if self.keep_first < 0 or (self.keep_first and self.window is None):
+            raise ValueError("first tokens are kept in sight beside a window")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         self.position = None
         if position is not None:
@@ -82,7 +90,8 @@ class GroupedQueryAttention(Mixer):
 
     def cache_spec(self):
         return CacheSpec("paged_kv", heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window,
-                         chunk=self.chunk, value_dim=None if self.value_dim == self.head_dim else self.value_dim)
+                         chunk=self.chunk, value_dim=None if self.value_dim == self.head_dim else self.value_dim,
+                         keep_first=self.keep_first)
 
     def tensor_decls(self):
         h, d, dv = self.hidden_size, self.head_dim, self.value_dim
@@ -126,7 +135,7 @@ class GroupedQueryAttention(Mixer):
         for q, kv in spans:  # scores and weighted values: 4 D operations per (query head, visible key)
             first = kv - q
             if self.window:
-                pairs = sum(min(first + i + 1, self.window) for i in range(q))
+                pairs = sum(min(first + i + 1, self.window + self.keep_first) for i in range(q))
             elif self.chunk:
                 pairs = sum((first + i) % self.chunk + 1 for i in range(q))
             else:
@@ -158,6 +167,10 @@ class GroupedQueryAttention(Mixer):
             more["chunk"] = self.chunk
         if self.softcap is not None:
             more["softcap"] = self.softcap
+        if self.keep_first:
+            more["keep_first"] = self.keep_first
+        if self.sink:
+            more["sink"] = True
         gate_width = nq * dv if self.output_gate else 0
         if gate_width:
             # the gate's columns stay where the product put them: the attention reads them there

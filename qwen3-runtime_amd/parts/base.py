@@ -175,6 +175,17 @@ class StreamUpdate:
 
 
 @dataclass
+class NormedUpdate:
+    """A sub-layer output that joins the residual stream through a norm of its own:
+    ``x <- x + y / rms(y) * weight`` (``rms`` with ``eps`` inside the root). Like a plain ``delta``
+    it is applied by the norm that comes next, which also normalises the sum."""
+
+    y: torch.Tensor       # [T, H], or float32 planes [P, T, H] whose sum it is
+    weight: torch.Tensor  # float32 [H]
+    eps: float
+
+
+@dataclass
 class GroupView:
     """One cache group's view of this step's batch (device tensors).
 
@@ -190,6 +201,8 @@ class GroupView:
     slots: torch.Tensor
     # keys are kept for the chunk of this many positions that the newest token lies in
     chunk: int | None = None
+    # beside a window, the sequence's first tokens stay in sight (and their pages in the table)
+    keep_first: int = 0
 
 
 @dataclass

@@ -1,5 +1,5 @@
 """Arrangements of a layer's parts: the pre-norm residual block, over one residual stream or
-over several (hyper-connections).
+over several (hyper-connections), and the block with a norm on both sides of each sub-layer.
 
 ``x += mixer(norm_in(x)); x += feed_forward(norm_post(x))``: the form the
 reference's oracle writes (tests/cpu/reference_qwen3.py:79-110) and its model
@@ -12,7 +12,7 @@ with the norm that follows it without a block knowing its neighbour.
 from __future__ import annotations
 
 from ..registry import register_part
-from .base import Block, StreamUpdate
+from .base import Block, NormedUpdate, StreamUpdate
 from .plan import TensorDecl
 
 
@@ -37,6 +37,37 @@ class PreNormBlock(Block):
             return residual, mixed
         x = self.norm_post.forward(ctx, residual, mixed)
         return residual, self.feed_forward.forward(ctx, x)
+
+
+@register_part("block", "sandwich_norm")
+class SandwichNormBlock(Block):
+    """A norm on both sides of each sub-layer: ``x += norm_after(mixer(norm_in(x)))``, then
+    ``x += norm_after_ff(feed_forward(norm_post(x)))``. The norm behind a sub-layer goes with its
+    output as a ``NormedUpdate``, so that the norm in front of the next sub-layer applies it, adds
+    and normalises in one pass over the stream."""
+
+    norm_names = ("input", "after_mixer", "post_mixer", "after_ff")
+
+    def __init__(self, mixer, feed_forward, norms, tensors=None):
+        super().__init__(tensors)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norm_in, self.after_mixer = norms["input"], norms["after_mixer"]
+        self.norm_post, self.after_ff = norms.get("post_mixer"), norms.get("after_ff")
+        if feed_forward is not None and (self.norm_post is None or self.after_ff is None):
+            raise ValueError("a feed-forward comes with the norms in front of it and behind it")
+
+    def children(self):
+        return tuple(p for p in (self.norm_in, self.mixer, self.after_mixer, self.norm_post, self.feed_forward,
+                                 self.after_ff) if p is not None)
+
+    def forward(self, ctx, residual, delta, cache):
+        x = self.norm_in.forward(ctx, residual, delta)
+        pending = NormedUpdate(self.mixer.forward(ctx, x, cache), self.after_mixer.weight, self.after_mixer.eps)
+        if self.feed_forward is None:
+            return residual, pending
+        x = self.norm_post.forward(ctx, residual, pending)
+        return residual, NormedUpdate(self.feed_forward.forward(ctx, x), self.after_ff.weight, self.after_ff.eps)
 
 
 @register_part("block", "hyper_connections")

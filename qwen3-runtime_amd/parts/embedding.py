@@ -4,6 +4,8 @@
 ``logits = x W^T`` where ``W`` is the embedding table when the head is tied,
 no bias and no scaling of logits (reference: qwen3_runtime/models/qwen3.py:265-266).
 The embedding starts the float32 residual stream; logits come out in float32.
+Either takes a constant ``scale`` (1 by default): the embedding's rows times it, in float32, and
+the float32 logits times it.
 """
 
 from __future__ import annotations
@@ -17,10 +19,11 @@ from .plan import TensorDecl
 class TokenEmbedding(Part):
     role = "embedding"
 
-    def __init__(self, vocab_size: int, hidden_size: int, tensors=None):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, tensors=None):
         super().__init__(tensors)
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
+        self.scale = float(scale)
         self.weight = None
 
     def tensor_decls(self):
@@ -30,6 +33,8 @@ class TokenEmbedding(Part):
         self.weight = fetch.matrix(self._name("weight"))
 
     def forward(self, ctx, ids):
+        if self.scale != 1.0:
+            return ctx.ops.embed(ids, self.weight, scale=self.scale)
         return ctx.ops.embed(ids, self.weight)
 
     def step_cost(self, spans, rows, elem_bytes):
@@ -44,10 +49,11 @@ class LinearHead(Part):
 
     role = "head"
 
-    def __init__(self, vocab_size: int, hidden_size: int, tensors=None):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, tensors=None):
         super().__init__(tensors)
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
+        self.scale = float(scale)
         self.weight = None
 
     def tensor_decls(self):
@@ -57,7 +63,8 @@ class LinearHead(Part):
         self.weight = fetch.matrix(self._name("weight"))
 
     def forward(self, ctx, x):
-        return ctx.ops.linear(x, self.weight, out_f32=True)
+        logits = ctx.ops.linear(x, self.weight, out_f32=True)
+        return logits if self.scale == 1.0 else ctx.ops.scale(logits, self.scale)
 
     def step_cost(self, spans, rows, elem_bytes):
         # the whole matrix, multiplied with the wanted rows only

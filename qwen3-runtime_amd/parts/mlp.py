@@ -1,9 +1,11 @@
-"""Dense gated feed-forward (SwiGLU).
+"""Dense feed-forwards: gated (SwiGLU), and plain with an activation between two matrices.
 
 ``down( silu(gate(x)) * up(x) )`` with gate and up as one fused matrix whose
 rows are gate's followed by up's (reference: qwen3_runtime/models/qwen3.py:130-138,
 qwen3_runtime/utils/loader.py:51-53); ``silu(g) = g * sigmoid(g)``
 (reference: qwen3_runtime/layers/ops.py:23-25), evaluated in float32 here.
+
+``act_mlp``: ``down( act(up(x)) )`` without a gate; ``act`` is ``relu2`` (the square of relu), in float32.
 """
 
 from __future__ import annotations
@@ -36,4 +38,30 @@ class SwiGLU(FeedForward):
 
     def forward(self, ctx, x):
         act = ctx.ops.gated_linear(x, self.gate_up)
+        return ctx.ops.linear_for_residual(act, self.down)
+
+
+@register_part("feed_forward", "act_mlp")
+class ActMLP(FeedForward):
+    """``tensors``: ``up``, ``down``."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu2", tensors=None):
+        super().__init__(tensors)
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        if activation not in ("relu2",):
+            raise ValueError(f"unknown activation {activation!r} (relu2)")
+        self.activation = activation
+        self.up = self.down = None
+
+    def tensor_decls(self):
+        h, i = self.hidden_size, self.intermediate_size
+        return [TensorDecl(self._name("up"), (i, h)), TensorDecl(self._name("down"), (h, i))]
+
+    def load(self, fetch):
+        self.up = fetch.matrix(self._name("up"))
+        self.down = fetch.matrix(self._name("down"))
+
+    def forward(self, ctx, x):
+        act = ctx.ops.unary_act(ctx.ops.linear(x, self.up), self.activation)
         return ctx.ops.linear_for_residual(act, self.down)

@@ -8,9 +8,11 @@ matrices lie in two tensors, ``[E, 2I, H]`` (gate rows, then up rows) and ``[E, 
 one launch serves every (token, chosen expert) pair.
 
 Options beyond that form. ``scoring="sigmoid"``: scores ``s = sigmoid(z)``; the ``top`` largest are
-chosen and weigh the experts' outputs as they are, not renormalised. ``groups`` and ``keep``: the
-experts form ``groups`` equal groups of neighbours, a group's score is the sum of its two largest
-scores, and only experts of the ``keep`` best groups can be chosen. ``activation="clamped"`` with
+chosen and weigh the experts' outputs as they are, not renormalised. ``scoring="softmax_all"``: scores
+``s = softmax(z)`` over all experts; the ``top`` largest are chosen and weigh the outputs as they are.
+``groups`` and ``keep``: the experts form ``groups`` equal groups of neighbours, a group's score is the
+sum of its two largest scores (``group_score="top2"``) or its largest score (``"max"``), and only
+experts of the ``keep`` best groups can be chosen. ``activation="clamped"`` with
 ``limit``: ``g = min(gate x, limit)``, ``u = clamp(up x, -limit, limit)``, ``y = g sigmoid(1.702 g) (u + 1)``
 in place of ``silu(g) u``. ``shared_size``: one more expert of that inner width (tensors
 ``shared_gate``, ``shared_up``, ``shared_down``; ``shared_limit`` its clamp) that every token passes
@@ -33,7 +35,7 @@ class RoutedSwiGLU(FeedForward):
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
                  router_bias: bool = True, scoring: str = "softmax_top", groups: int = 1, keep: int | None = None,
                  activation: str = "swiglu", limit: float = 0.0, shared_size: int | None = None,
-                 shared_limit: float | None = None, tensors=None):
+                 shared_limit: float | None = None, group_score: str = "top2", tensors=None):
         super().__init__(tensors)
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
@@ -42,9 +44,12 @@ class RoutedSwiGLU(FeedForward):
         if not 1 <= self.top <= self.num_experts:
             raise ValueError(f"each token takes {self.top} of {self.num_experts} experts")
         self.has_router_bias = bool(router_bias)
-        if scoring not in ("softmax_top", "sigmoid") or activation not in ("swiglu", "clamped"):
-            raise ValueError(f"unknown scoring {scoring!r} (softmax_top, sigmoid) or activation {activation!r} (swiglu, clamped)")
+        if scoring not in ("softmax_top", "sigmoid", "softmax_all") or activation not in ("swiglu", "clamped") \
+                or group_score not in ("top2", "max"):
+            raise ValueError(f"unknown scoring {scoring!r} (softmax_top, sigmoid, softmax_all), activation {activation!r} "
+                             f"(swiglu, clamped) or group score {group_score!r} (top2, max)")
         self.scoring, self.activation, self.limit = scoring, activation, float(limit)
+        self.group_score = group_score
         self.groups = int(groups)
         self.keep = self.groups if keep is None else int(keep)
         if self.groups < 1 or self.num_experts % self.groups or not 1 <= self.keep <= self.groups:
@@ -109,8 +114,9 @@ class RoutedSwiGLU(FeedForward):
         if plain:
             index, weight = ops.route_top(x, self.router, self.router_bias, self.top)
             return ops.moe_swiglu(x, self.gate_up, self.down, index, weight)
+        how = {"group_score": self.group_score} if self.group_score != "top2" else {}
         index, weight = ops.route_top(x, self.router, self.router_bias, self.top, scoring=self.scoring,
-                                      groups=self.groups, keep=self.keep)
+                                      groups=self.groups, keep=self.keep, **how)
         more = {"activation": self.activation, "limit": self.limit}
         if not self.shared_size:
             return ops.moe_swiglu(x, self.gate_up, self.down, index, weight, **more)

@@ -22,7 +22,7 @@ from __future__ import annotations
 import torch
 
 from ..registry import register_part
-from .base import Norm
+from .base import Norm, NormedUpdate
 from .plan import TensorDecl
 
 
@@ -63,6 +63,12 @@ class RMSNorm(Norm):
         if residual.dim() == 3:  # several streams
             return ctx.ops.mix_norm(residual, delta, self.read_all if read is None else read, self.weight,
                                     self.bias, self.eps, ctx.dtype, rows)
+        if isinstance(delta, NormedUpdate):
+            # a sub-layer output that is normed on its way into the stream
+            if self.has_bias or self.delta_scale != 1.0:
+                raise NotImplementedError("a normed update meets the plain RMS norm only")
+            return ctx.ops.add_rmsnorm(residual, delta.y, self.weight, self.eps, ctx.dtype, rows,
+                                       delta_norm=(delta.weight, delta.eps))
         if self.has_bias:
             return ctx.ops.mix_norm(residual, delta, None, self.weight, self.bias, self.eps, ctx.dtype, rows)
         if self.delta_scale != 1.0:

@@ -72,7 +72,8 @@ class CacheSpec:
     """What one cache owner keeps between steps.
 
     ``kind == "paged_kv"``: keys and values for every token (or the last
-    ``window`` tokens, or, with ``chunk``, the tokens of the chunk of ``chunk``
+    ``window`` tokens, beside which the sequence's first ``keep_first`` stay for good, or,
+    with ``chunk``, the tokens of the chunk of ``chunk``
     positions, counted from position 0, that the newest token lies in),
     ``heads`` x ``head_dim`` keys and ``heads`` x ``value_dim``
     values (``head_dim`` when None), held in pages; the values transposed within a
@@ -91,10 +92,13 @@ class CacheSpec:
     value_dim: int | None = None
     streams: tuple[PagedStream, ...] = ()
     chunk: int | None = None
+    keep_first: int = 0
 
     def __post_init__(self) -> None:
         if self.window is not None and self.chunk is not None:
             raise ValueError("a cache keeps a window of keys or a chunk of them, not both")
+        if self.keep_first < 0 or (self.keep_first and self.window is None):
+            raise ValueError("first tokens are kept beside a window, and their number is not negative")
         for name in ("window", "chunk"):
             if getattr(self, name) is not None and getattr(self, name) < 1:
                 raise ValueError(f"{name} must be positive, got {getattr(self, name)}")
@@ -121,7 +125,7 @@ class CacheSpec:
     def group_key(self) -> tuple:
         """Caches with equal keys share pages' geometry and lifetime, hence a pool."""
         if self.paged:
-            return ("paged", self.page_streams(), self.window, self.chunk)
+            return ("paged", self.page_streams(), self.window, self.chunk, self.keep_first)
         return ("state", tuple(self.shape), self.dtype)
 
 

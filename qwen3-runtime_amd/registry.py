@@ -136,3 +136,4 @@ def _load_builtin() -> None:
     from .models import qwen3  # noqa: F401  (registers Qwen3ForCausalLM; its presets come first)
     from .models import deginex  # noqa: F401  (registers Deginex)
     from .models import zisedra  # noqa: F401  (registers Zisedra)
+    from .models import roserax  # noqa: F401  (registers Roserax)

@@ -17,13 +17,19 @@ import math
 import torch
 
 
-def embed(ids, table):
-    return table[ids.long()].to(torch.float32)
+def embed(ids, table, scale=1.0):
+    x = table[ids.long()].to(torch.float32)
+    return x if scale == 1.0 else x * scale
 
 
-def add_rmsnorm(residual, delta, weight, eps, out_dtype, rows=None, compute=torch.float32, delta_scale=1.0):
+def add_rmsnorm(residual, delta, weight, eps, out_dtype, rows=None, compute=torch.float32, delta_scale=1.0,
+                delta_norm=None):
     if delta is not None and delta.dim() == 3:
         delta = delta.to(residual.dtype).sum(0)
+    if delta_norm is not None:  # the pending output is normed on its way into the stream
+        after_w, after_eps = delta_norm
+        d = delta.to(torch.float32)
+        delta = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + after_eps) * after_w
     if delta is not None and delta_scale != 1.0:
         delta = delta.to(residual.dtype) * delta_scale
     if delta is not None:
@@ -110,8 +116,10 @@ def gather_kv(k_cache, v_cache, table_row, lo, hi, page_size):
 
 def paged_attention(q, k_cache, v_cache, cu_q, kv_lens, block_table, page_size, nq, nkv, d,
                     scale, window=None, compute=torch.float32, round_probs=False, chunk=None, softcap=None,
-                    value_dim=None, gate=None):
-    """q [T, nq*D] -> [T, nq*Dv]. Query row i of a sequence sits at position
+                    value_dim=None, gate=None, keep_first=0, sink=False):
+    """q [T, nq*D] -> [T, nq*Dv]. ``keep_first``: beside a window the sequence's first tokens stay
+    visible; ``sink``: one more term of score 0 in the softmax's denominator.
+    Query row i of a sequence sits at position
     kv_len - q_len + i and sees keys j <= its position (and > position - window, or, with
     ``chunk``, in its own chunk of positions). ``softcap``: scores become cap * tanh(score / cap).
     ``gate`` [T, nq*Dv]: the output is multiplied by its sigmoid."""
@@ -125,25 +133,42 @@ def paged_attention(q, k_cache, v_cache, cu_q, kv_lens, block_table, page_size, 
         if q_len == 0 or kv_len == 0:
             continue
         first_pos = kv_len - q_len
-        lo = 0 if window is None else max(0, first_pos - window + 1)
+        lo = 0 if window is None or keep_first else max(0, first_pos - window + 1)
         if chunk is not None:
             lo = first_pos - first_pos % chunk
-        k, v = gather_kv(k_cache, v_cache, block_table[s], lo, kv_len, page_size)
-        k = k.to(compute).repeat_interleave(g, dim=1)
-        v = v.to(compute).repeat_interleave(g, dim=1)
-        qs = q[a:b].reshape(q_len, nq, d).to(compute)
-        scores = torch.einsum("qhd,khd->hqk", qs, k) * scale
         qpos = torch.arange(first_pos, kv_len, device=q.device)[:, None]
         kpos = torch.arange(lo, kv_len, device=q.device)[None, :]
         ok = kpos <= qpos
         if window is not None:
-            ok = ok & (kpos > qpos - window)
+            ok = ok & ((kpos > qpos - window) | (kpos < keep_first))
         if chunk is not None:
             ok = ok & (kpos // chunk == qpos // chunk)
+        if keep_first and window is not None:
+            # the pages between the kept tokens and the window may be gone: read only what some row sees
+            idx = ok.any(dim=0).nonzero()[:, 0]
+            pos_seen = kpos[0, idx]
+            pages = block_table[s].long()[pos_seen // page_size]
+            if (pages < 0).any():
+                raise AssertionError("attention reads a position whose page was given back")
+            k = torch.zeros((kv_len - lo, nkv, d), dtype=k_cache.dtype, device=q.device)
+            v = torch.zeros((kv_len - lo, nkv, dv), dtype=v_cache.dtype, device=q.device)
+            k[idx] = k_cache[pages, :, pos_seen % page_size, :]
+            v[idx] = v_cache[pages, :, :, pos_seen % page_size]
+        else:
+            k, v = gather_kv(k_cache, v_cache, block_table[s], lo, kv_len, page_size)
+        k = k.to(compute).repeat_interleave(g, dim=1)
+        v = v.to(compute).repeat_interleave(g, dim=1)
+        qs = q[a:b].reshape(q_len, nq, d).to(compute)
+        scores = torch.einsum("qhd,khd->hqk", qs, k) * scale
         if softcap is not None:
             scores = softcap * torch.tanh(scores / softcap)
         scores = scores.masked_fill(~ok, float("-inf"))
-        probs = torch.softmax(scores, dim=-1)
+        if sink:
+            m = torch.clamp(scores.amax(dim=-1, keepdim=True), min=0.0)
+            e = torch.exp(scores - m)
+            probs = e / (torch.exp(-m) + e.sum(dim=-1, keepdim=True))
+        else:
+            probs = torch.softmax(scores, dim=-1)
         if round_probs:
             probs = probs.to(q.dtype).to(compute)
         ctx = torch.einsum("hqk,khd->qhd", probs, v).reshape(q_len, nq * dv)
@@ -187,26 +212,27 @@ def mix_norm(streams, update, read, weight, bias, eps, out_dtype, rows=None, com
     return y.to(out_dtype)
 
 
-def route_top(x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None):
+def route_top(x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None, group_score="top2"):
     """float32 logits x W^T + b; the ``top`` largest per token (ties: the lower index first) and
     the softmax over those alone. Returns (int32 [T, top], float32 [T, top]). With sigmoid scoring
     the scores are the weights; with groups only the best ``keep`` groups' experts can be chosen."""
     logits = x.to(torch.float32) @ router.to(torch.float32).T
     if router_bias is not None:
         logits = logits + router_bias.to(torch.float32)
-    values = torch.sigmoid(logits) if scoring == "sigmoid" else logits
+    values = torch.sigmoid(logits) if scoring == "sigmoid" else \
+        torch.softmax(logits, dim=-1) if scoring == "softmax_all" else logits
     pick = values
     if groups > 1 and keep is not None and keep < groups:
         t, e = values.shape
         per = e // groups
         g = values.view(t, groups, per)
-        gscore = torch.topk(g, min(2, per), dim=-1).values.sum(-1)
+        gscore = g.amax(dim=-1) if group_score == "max" else torch.topk(g, min(2, per), dim=-1).values.sum(-1)
         stay = torch.zeros(t, groups, dtype=torch.bool, device=x.device)
         stay.scatter_(1, torch.topk(gscore, keep, dim=-1).indices, True)
         pick = torch.where(stay[:, :, None].expand(t, groups, per).reshape(t, e), values,
                            torch.full_like(values, float("-inf")))
     best, index = torch.topk(pick, top, dim=-1)
-    return index.to(torch.int32), best if scoring == "sigmoid" else torch.softmax(best, dim=-1)
+    return index.to(torch.int32), best if scoring != "softmax_top" else torch.softmax(best, dim=-1)
 
 
 def gated(g, u, activation="swiglu", limit=0.0):
@@ -330,17 +356,128 @@ def argmax(logits):
     return torch.argmax(logits, dim=-1).to(torch.int32)
 
 
+def rotate_half_copy(x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq):
+    """For every token and head copy ``width`` elements from ``x[t, h * in_stride + in_offset ...]`` to
+    ``out[t, h * out_stride + out_offset ...]``, the first ``2 len(freq)`` of them turned: element i
+    against element i + len(freq), by ``position * freq[i]`` (float32 angles)."""
+    t = x.shape[0]
+    src = x.view(t, heads, in_stride)[:, :, in_offset: in_offset + width].to(torch.float32)
+    n = 0 if freq is None else freq.numel()
+    if n:
+        ang = positions.to(torch.float32)[:, None] * freq.to(torch.float32)[None, :]
+        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        u, v = src[..., :n], src[..., n: 2 * n]
+        src = torch.cat([u * cos - v * sin, v * cos + u * sin, src[..., 2 * n:]], dim=-1)
+    out.view(t, heads, out_stride)[:, :, out_offset: out_offset + width] = src.to(out.dtype)
+    return out
+
+
+def rmsnorm_columns(y, first, width, weight, eps):
+    x = y[:, first: first + width].to(torch.float32)
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight).to(y.dtype)
+
+
+def latent_store(y, first, rank, rot_dim, weight, eps, positions, freq, k_cache, v_cache, slots, page_size):
+    """Columns ``first .. first + rank`` of ``y`` RMS-normed (the latent) and the ``rot_dim`` behind them
+    rotated: the key row ``[c | k_rot]`` and the value row ``[c | 0]`` of one key/value head."""
+    t = y.shape[0]
+    c = rmsnorm_columns(y, first, rank, weight, eps).to(torch.float32)
+    rot = torch.empty((t, rot_dim), dtype=torch.float32, device=y.device)
+    rotate_half_copy(y[:, first + rank: first + rank + rot_dim].contiguous(), rot_dim, 0, rot, rot_dim, 0, 1, rot_dim,
+                     positions, freq)
+    k = torch.cat([c, rot], dim=1)[:, None, :]
+    v = torch.cat([c, torch.zeros_like(rot)], dim=1)[:, None, :]
+    kv_store(k, v, k_cache, v_cache, slots, page_size)
+
+
+def heads_linear(x, in_stride, in_offset, w, out, out_stride, out_offset, compute=torch.float32):
+    """Per head h: out[t, h * out_stride + out_offset + n] = sum_k w[h, n, k] x[t, h * in_stride + in_offset + k]."""
+    t = x.shape[0]
+    heads, n, k = w.shape
+    src = x.view(t, heads, in_stride)[:, :, in_offset: in_offset + k].to(compute)
+    res = torch.einsum("thk,hnk->thn", src, w.to(compute))
+    out.view(t, heads, out_stride)[:, :, out_offset: out_offset + n] = res.to(out.dtype)
+    return out
+
+
+def retention_prepare(y, heads, dim, vdim, positions, freq, k_scale):
+    """float32 [T, 2 heads dim + heads vdim]: queries and keys rotated (keys then scaled), values as they are."""
+    t = y.shape[0]
+    out = torch.empty((t, 2 * heads * dim + heads * vdim), dtype=torch.float32, device=y.device)
+    src = y[:, : 2 * heads * dim].contiguous()
+    rotate_half_copy(src, dim, 0, out[:, : 2 * heads * dim], dim, 0, 2 * heads, dim, positions, freq)
+    out[:, heads * dim: 2 * heads * dim] *= k_scale
+    out[:, 2 * heads * dim:] = y[:, 2 * heads * dim: 2 * heads * dim + heads * vdim].to(torch.float32)
+    return out
+
+
+def retention_rule(qkv, decay, state, cu_q, slots, heads, dim, vdim):
+    """S <- decay S + k v^T; o = S^T q, per sequence and head from the slot's state [slots, heads, vdim, dim]."""
+    t = qkv.shape[0]
+    q = qkv[:, : heads * dim].view(t, heads, dim)
+    k = qkv[:, heads * dim: 2 * heads * dim].view(t, heads, dim)
+    v = qkv[:, 2 * heads * dim:].view(t, heads, vdim)
+    out = torch.empty((t, heads, vdim), dtype=torch.float32, device=qkv.device)
+    for s in range(len(cu_q) - 1):
+        slot = int(slots[s])
+        st = state[slot].clone()  # [heads, vdim, dim]
+        for i in range(int(cu_q[s]), int(cu_q[s + 1])):
+            st = st * decay[:, None, None] + v[i][:, :, None] * k[i][:, None, :]
+            out[i] = torch.einsum("hvd,hd->hv", st, q[i])
+        state[slot] = st
+    return out
+
+
+def unary_act(x, kind):
+    if kind != "relu2":
+        raise ValueError(kind)
+    return torch.relu(x.to(torch.float32)).pow(2).to(x.dtype)
+
+
 class TorchOps:
     """The engine's op interface over the functions above (tests only)."""
 
     def __init__(self, compute=torch.float32):
         self.compute = compute
 
-    def embed(self, ids, table):
-        return embed(ids, table)
+    def embed(self, ids, table, scale=1.0):
+        return embed(ids, table, scale)
 
-    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None, delta_scale=1.0):
-        return add_rmsnorm(residual, delta, weight, eps, out_dtype, rows, self.compute, delta_scale)
+    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None, delta_scale=1.0, delta_norm=None):
+        return add_rmsnorm(residual, delta, weight, eps, out_dtype, rows, self.compute, delta_scale, delta_norm)
+
+    def scale(self, x, factor):
+        return x.mul_(factor)
+
+    def new_rows(self, t, width, dtype, device):
+        return torch.empty((t, width), dtype=dtype, device=device)
+
+    def rmsnorm_columns(self, y, first, width, weight, eps):
+        return rmsnorm_columns(y, first, width, weight, eps)
+
+    def latent_store(self, y, first, rank, rot_dim, weight, eps, positions, freq, cache):
+        if cache is not None:
+            latent_store(y, first, rank, rot_dim, weight, eps, positions, freq, cache.k, cache.v, cache.group.slots,
+                         cache.group.page_size)
+
+    def heads_linear(self, x, in_stride, in_offset, w, out, out_stride, out_offset):
+        return heads_linear(x, in_stride, in_offset, w, out, out_stride, out_offset, self.compute)
+
+    def rotate_half(self, x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq):
+        return rotate_half_copy(x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq)
+
+    def sigmoid_gate(self, out, gate):
+        out.copy_((out.to(torch.float32) * torch.sigmoid(gate.to(torch.float32))).to(out.dtype))
+        return out
+
+    def retention_prepare(self, y, heads, dim, vdim, positions, freq, k_scale):
+        return retention_prepare(y, heads, dim, vdim, positions, freq, k_scale)
+
+    def retention_rule(self, ctx, qkv, decay, state, heads, dim, vdim):
+        return retention_rule(qkv, decay, state, ctx.cu_q, ctx.state_slots, heads, dim, vdim)
+
+    def unary_act(self, x, kind):
+        return unary_act(x, kind)
 
     def norm_mean(self, ya, wa, yb, wb, eps):
         return norm_mean(ya, wa, yb, wb, eps)
@@ -391,8 +528,8 @@ class TorchOps:
     def mix_norm(self, streams, update, read, weight, bias, eps, out_dtype, rows=None):
         return mix_norm(streams, update, read, weight, bias, eps, out_dtype, rows, self.compute)
 
-    def route_top(self, x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None):
-        return route_top(x, router, router_bias, top, scoring, groups, keep)
+    def route_top(self, x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None, group_score="top2"):
+        return route_top(x, router, router_bias, top, scoring, groups, keep, group_score)
 
     def moe_swiglu(self, x, gate_up, down, index, weight, activation="swiglu", limit=0.0):
         return moe_swiglu(x, gate_up, down, index, weight, self.compute, activation, limit)
@@ -411,10 +548,10 @@ class TorchOps:
         kv_store(k, v, cache.k, cache.v, cache.group.slots, cache.group.page_size)
 
     def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window, chunk=None, softcap=None, value_dim=None,
-                        gate=None):
+                        gate=None, keep_first=0, sink=False):
         return paged_attention(q, cache.k, cache.v, ctx.cu_q, ctx.kv_lens, cache.group.block_table,
                                cache.group.page_size, nq, nkv, d, scale, window, self.compute, chunk=chunk,
-                               softcap=softcap, value_dim=value_dim, gate=gate)
+                               softcap=softcap, value_dim=value_dim, gate=gate, keep_first=keep_first, sink=sink)
 
     def swiglu(self, gate_up):
         return swiglu(gate_up, self.compute)
