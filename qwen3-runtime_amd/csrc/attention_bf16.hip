@@ -24,8 +24,9 @@
 // exponent's argument); probabilities are rounded to bfloat16 for the second
 // product, accumulation is float32. Key j is visible to the row at position p
 // iff first_seen(p) <= j <= p: the first key a row sees is 0, or p - window + 1 with a window, or
-// the first position of p's chunk (p - p % chunk) with a mask of chunks. With a score cap the
-// scaled scores become cap * tanh(score / cap) before the softmax.
+// the first position of p's chunk (p - p % chunk) with a mask of chunks; beside a window the first
+// keep_first keys of the sequence are visible too. With a score cap the scaled scores become
+// cap * tanh(score / cap) before the softmax; with a sink the denominator has one more term, 1.
 #include "common.h"
 #include <math.h>
 
@@ -97,6 +98,15 @@ struct AttnTileArgs {
   // q, k and v, say). Applied where the output is written: here, or in the merge of key splits.
   const bf16_t* gate;
   long gate_stride;
+  // Beside a window: the sequence's first keep_first keys stay visible to every later query (their
+  // pages stay in the block table; those between them and the window may be gone, and no load goes
+  // there). A wave walks them in a pass of its own, [0, min(keep_first, first key of its window)),
+  // before the window's blocks; inside the window's blocks a key below a row's own window is
+  // visible if it is a kept one and not one of that first pass.
+  int keep_first;
+  // 1: the softmax's denominator has one more term of score 0 and no value,
+  // p_j = exp(s_j) / (1 + sum exp(s_j)): added where the sums are final (here, or in the merge).
+  int sink;
 };
 
 // The first key position that the query at position p sees. It does not fall as p grows, so for a
@@ -175,6 +185,7 @@ __device__ __forceinline__ float row_max4(float x) {
 
 __device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t* vv, bool masked, int base,
                                             int quad, bool row_valid, int qpos, int window, int chunk,
+                                            int keep, int lo_min,
                                             float scale_log2, float& m, float& l, f32x4_t* o) {
   float s[8];
 #pragma unroll
@@ -184,7 +195,7 @@ __device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t*
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int key = base + 8 * quad + e;
-      const bool vis = row_valid && key <= qpos && key >= lo_row;
+      const bool vis = row_valid && key <= qpos && (key >= lo_row || (key < keep && key >= lo_min));
       s[e] = vis ? s[e] : -INFINITY;
     }
   }
@@ -222,6 +233,7 @@ __device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t*
 template <int RT>
 __device__ __forceinline__ void tiles_update(const f32x4_t (*sc)[2], const bf16x8_t* vv, unsigned whole, int base,
                                              int quad, const bool* row_valid, const int* qpos, int window, int chunk,
+                                             int keep, int lo_min,
                                              float scale_log2, float* m, float* l, f32x4_t (*o)[DB]) {
   // whole: bit t says that every row of tile t sees all 32 keys (one scalar for the wave: an
   // array of flags went through vector registers, a dozen instructions per block of keys)
@@ -237,7 +249,8 @@ __device__ __forceinline__ void tiles_update(const f32x4_t (*sc)[2], const bf16x
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int key = base + 8 * quad + e;
-        const bool vis = ((whole >> t) & 1) || (row_valid[t] && key <= qpos[t] && key >= lo_row);
+        const bool vis = ((whole >> t) & 1) ||
+                         (row_valid[t] && key <= qpos[t] && (key >= lo_row || (key < keep && key >= lo_min)));
         s[t][e] = vis ? s[t][e] : -INFINITY;
       }
     }
@@ -330,6 +343,55 @@ __device__ __forceinline__ void block_load(const AttnTileArgs& a, int kvh, int b
     blk.v[i] = ONCE ? load_once8(vp + (size_t)16 * i * ps) : *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
 }
 
+// The kept first keys [0, kend) of a sequence against the RT tiles of a wave, every row of which
+// sees all of them (kend <= the first key of the wave's window): blocks of 32 keys straight from
+// the pages, a handful at most, before (or after) the window's blocks. Loads are clamped into
+// [0, kend - 1], which lies in pages the table keeps.
+template <int RT, bool P2>
+__device__ __forceinline__ void kept_keys_pass(const AttnTileArgs& a, const int* __restrict__ table, int kvh, int kend,
+                                               int r16, int quad, const bool* row_valid,
+                                               const bf16x8_t (*qreg)[KFULL > 0 ? KFULL : 1], const bf16x8_t* qtail,
+                                               float* m, float* l, f32x4_t (*o)[DB]) {
+  for (int base = 0; base < kend; base += 32) {
+    int pg[3];
+    KvBlock blk;
+    block_pages<P2>(table, base, 0, kend - 1, a.page_size, r16, quad, pg);
+    block_load<P2>(a, kvh, base, 0, kend - 1, r16, quad, pg, blk);
+    const bool partial = base + 31 > kend - 1;
+    if (partial) {
+      const int keep = kend - (base + 8 * quad);
+#pragma unroll
+      for (int i = 0; i < DB; ++i) blk.v[i] = keep_first(blk.v[i], keep);
+    }
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      f32x4_t sc[2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < KFULL; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[kb][i], qreg[t][i], acc, 0, 0, 0);
+        if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kt[kb], qtail[t], acc, 0, 0, 0);
+        sc[kb] = acc;
+      }
+      if (a.cap_in > 0.f) cap_scores(sc, a.cap_in, a.cap_out);
+      // as a causal row at position kend - 1: all keys up to there, none after
+      tile_update(sc, blk.v, partial, base, quad, row_valid[t], kend - 1, 0, 0, 0, 0, a.scale_log2, m[t], l[t], o[t]);
+    }
+  }
+}
+
+// The sink joins a row's final sum: one more term of score 0 under the row's reference m (scaled
+// base-2 units); the accumulator shrinks with the sum if the reference has to rise to 0.
+__device__ __forceinline__ void add_sink(float& m, float& l_total, f32x4_t* o) {
+  const float m_new = max2(m, 0.f);
+  const float corr = __builtin_amdgcn_exp2f(m - m_new);  // m = -inf: 0
+  l_total = l_total * corr + __builtin_amdgcn_exp2f(-m_new);
+#pragma unroll
+  for (int i = 0; i < DB; ++i) o[i] *= corr;
+  m = m_new;
+}
+
 // General kernel (prompt portions and mixed batches). A wave owns RT tiles of 16
 // rows each, 16 * RT consecutive rows of the sequence's row matrix; a block is
 // four waves, 64 * RT rows. The keys and values of a block of 32 keys are read
@@ -399,6 +461,9 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
     for (int i = 0; i < DB; ++i) o[t][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   }
 
+  if (a.keep_first > 0 && split == 0)
+    kept_keys_pass<RT, P2>(a, table, kvh, min(a.keep_first, lo), r16, quad, row_valid, qreg, qtail, m, l, o);
+
   // page numbers are looked up one block ahead of the loads that need them; all loads are
   // unconditional (clamped), see block_pages / block_load
   if (b0 < b1) {
@@ -433,7 +498,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
         // every row of the tile sees the whole block unless it touches the diagonal or the edge of
         // a window or a chunk
         const bool whole = base + 31 <= tile_pos_min[t] && base >= tile_lo_max[t];
-        tile_update(s, blk.v, !whole, base, quad, row_valid[t], qpos[t], a.window, a.chunk, a.scale_log2, m[t], l[t], o[t]);
+        tile_update(s, blk.v, !whole, base, quad, row_valid[t], qpos[t], a.window, a.chunk, a.keep_first, lo, a.scale_log2, m[t], l[t], o[t]);
       }
 #pragma unroll
       for (int i = 0; i < 3; ++i) pg[i] = pg_next[i];
@@ -446,6 +511,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
     if (!row_valid[t]) continue;
+    if (a.sink && a.num_splits == 1) add_sink(m[t], lt, o[t]);
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     if (a.num_splits == 1) {
       bf16_t* op = a.out + row_index[t] * D;
@@ -495,12 +561,12 @@ constexpr int KROW = D % 32 == 0 ? D + 16 : D;  // elements per key row in LDS
 constexpr float LAZY = 8.0f;
 
 __device__ __forceinline__ void tile_mask(f32x4_t sc[2], int base, int quad, bool row_valid, int qpos, int window,
-                                          int chunk) {
+                                          int chunk, int keep, int lo_min) {
   const int lo_row = first_seen(qpos, window, chunk);
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const int key = base + 8 * quad + e;
-    const bool vis = row_valid && key <= qpos && key >= lo_row;
+    const bool vis = row_valid && key <= qpos && (key >= lo_row || (key < keep && key >= lo_min));
     sc[e >> 2][e & 3] = vis ? sc[e >> 2][e & 3] : -INFINITY;
   }
 }
@@ -605,10 +671,12 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
   const int per = (all_b1 - all_b0 + a.num_splits - 1) / a.num_splits;
   const int b0 = all_b0 + split * per, b1 = min(all_b1, b0 + per);
   int wb0 = b1, wb1 = b0;  // this wave's blocks: none unless it has rows
+  int lo_w = lo;           // the first key of this wave's window
   if (wave_has_rows) {
     const int row_last = min(row0 + 16 * RT - 1, n_rows - 1);
     const int pos_min = first_pos + row0 / g, pos_max = first_pos + row_last / g;
-    wb0 = max(0, first_seen(pos_min, a.window, a.chunk)) >> 5;
+    lo_w = max(0, first_seen(pos_min, a.window, a.chunk));
+    wb0 = lo_w >> 5;
     wb1 = min((pos_max >> 5) + 1, b1);  // not into the next split's blocks
   }
 
@@ -621,6 +689,9 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
 #pragma unroll
     for (int i = 0; i < DB; ++i) o[t][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   }
+
+  if (a.keep_first > 0 && split == 0 && grp == 0 && wave_has_rows)
+    kept_keys_pass<RT, P2>(a, table, kvh, min(a.keep_first, lo_w), r16, quad, row_valid, qreg, qtail, m, l, o);
 
   // Who fetches what. A block of 32 keys is four groups of 8 consecutive keys, one per wave.
   // Pages hold a multiple of 8 keys, so a group lies in one page: the wave needs ONE block-table
@@ -737,11 +808,11 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
         const bool jumps = mx0 * a.scale_log2 > m[0] + LAZY || mx1 * a.scale_log2 > m[1] + LAZY;
         if (edge || __any(jumps)) {
           if (!sees_all(0)) {
-            tile_mask(sc0, base, quad, row_valid[0], qpos[0], a.window, a.chunk);
+            tile_mask(sc0, base, quad, row_valid[0], qpos[0], a.window, a.chunk, a.keep_first, lo_w);
             mx0 = lane_max(sc0);
           }
           if (!sees_all(1)) {
-            tile_mask(sc1, base, quad, row_valid[1], qpos[1], a.window, a.chunk);
+            tile_mask(sc1, base, quad, row_valid[1], qpos[1], a.window, a.chunk, a.keep_first, lo_w);
             mx1 = lane_max(sc1);
           }
           tile_move_reference(mx0, a.scale_log2, m[0], l[0], o[0]);
@@ -761,7 +832,7 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
           scores(t, sc[t]);
           whole |= (unsigned)sees_all(t) << t;
         }
-        tiles_update<RT>(sc, vv, whole, base, quad, row_valid, qpos, a.window, a.chunk, a.scale_log2, m, l, o);
+        tiles_update<RT>(sc, vv, whole, base, quad, row_valid, qpos, a.window, a.chunk, a.keep_first, lo_w, a.scale_log2, m, l, o);
       }
     }
   };
@@ -830,6 +901,7 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
     if (!row_valid[t] || !wave_has_rows || grp != 0) continue;
+    if (a.sink && a.num_splits == 1) add_sink(m[t], lt, o[t]);
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     if (a.num_splits == 1) {
       bf16_t* op = a.out + row_index[t] * D;
@@ -859,7 +931,7 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
 template <int MAX>
 __device__ __forceinline__ void merge_few(const float* __restrict__ part_o, const float* __restrict__ lse,
                                           bf16_t* __restrict__ out, int num_splits, size_t row,
-                                          const bf16_t* __restrict__ gate, long gate_stride, int nq) {
+                                          const bf16_t* __restrict__ gate, long gate_stride, int nq, int sink) {
   float ls[MAX], pv[2][MAX];
   const int d0 = min((int)threadIdx.x, D - 1), d1 = min((int)(threadIdx.x + blockDim.x), D - 1);
   const float g0 = gate_factor(gate, gate_stride, nq, row, d0), g1 = gate_factor(gate, gate_stride, nq, row, d1);
@@ -873,7 +945,8 @@ __device__ __forceinline__ void merge_few(const float* __restrict__ part_o, cons
   float mx = -INFINITY;
 #pragma unroll
   for (int s = 0; s < MAX; ++s) mx = fmaxf(mx, ls[s]);
-  float acc[2] = {0.f, 0.f}, wsum = 0.f;
+  if (sink) mx = fmaxf(mx, 0.f);  // the sink: one more part of weight 2^0 and no value
+  float acc[2] = {0.f, 0.f}, wsum = sink ? exp2f(-mx) : 0.f;
   if (mx != -INFINITY) {
 #pragma unroll
     for (int s = 0; s < MAX; ++s) {
@@ -895,21 +968,22 @@ __device__ __forceinline__ void merge_few(const float* __restrict__ part_o, cons
 // out[row] = sum_s 2^(lse_s - M) O_s / sum_s 2^(lse_s - M); empty splits weigh 0
 __global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse,
                                        bf16_t* __restrict__ out, int num_splits, const int* __restrict__ tokens,
-                                       int nq, const bf16_t* __restrict__ gate, long gate_stride) {
+                                       int nq, const bf16_t* __restrict__ gate, long gate_stride, int sink) {
   // rows are (token, query head); with a token list the grid walks the listed tokens' rows only
   const size_t row = tokens ? (size_t)tokens[blockIdx.x / nq] * nq + blockIdx.x % nq : blockIdx.x;
   const float* lse = part_lse + row * num_splits;
   if (num_splits <= 64 && D <= 2 * (int)blockDim.x) {
-    if (num_splits <= 8) merge_few<8>(part_o, lse, out, num_splits, row, gate, gate_stride, nq);
-    else if (num_splits <= 16) merge_few<16>(part_o, lse, out, num_splits, row, gate, gate_stride, nq);
-    else if (num_splits <= 32) merge_few<32>(part_o, lse, out, num_splits, row, gate, gate_stride, nq);
-    else merge_few<64>(part_o, lse, out, num_splits, row, gate, gate_stride, nq);
+    if (num_splits <= 8) merge_few<8>(part_o, lse, out, num_splits, row, gate, gate_stride, nq, sink);
+    else if (num_splits <= 16) merge_few<16>(part_o, lse, out, num_splits, row, gate, gate_stride, nq, sink);
+    else if (num_splits <= 32) merge_few<32>(part_o, lse, out, num_splits, row, gate, gate_stride, nq, sink);
+    else merge_few<64>(part_o, lse, out, num_splits, row, gate, gate_stride, nq, sink);
     return;
   }
   float mx = -INFINITY;
   for (int s = 0; s < num_splits; ++s) mx = fmaxf(mx, lse[s]);
+  if (sink) mx = fmaxf(mx, 0.f);
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float acc = 0.f, wsum = 0.f;
+    float acc = 0.f, wsum = sink ? exp2f(-mx) : 0.f;
     if (mx != -INFINITY) {
       const float* po = part_o + row * num_splits * D + d;
 #pragma unroll 8
@@ -988,7 +1062,7 @@ __global__ __launch_bounds__(256) void attention_work_list_kernel(AttnTileArgs a
 
 __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg, bf16x8_t qtail, int base, int lo,
                                               int pos_min, int pos_max, int quad, bool row_valid, int qpos,
-                                              int window, int chunk, float cap_in, float cap_out, float scale_log2,
+                                              int window, int chunk, int keep, float cap_in, float cap_out, float scale_log2,
                                               float& m, float& l, f32x4_t* o) {
   f32x4_t s[2];
 #pragma unroll
@@ -1010,7 +1084,7 @@ __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg
 #pragma unroll
     for (int i = 0; i < DB; ++i) blk.v[i] = keep_first(blk.v[i], keep);
   }
-  tile_update(s, blk.v, !whole, base, quad, row_valid, qpos, window, chunk, scale_log2, m, l, o);
+  tile_update(s, blk.v, !whole, base, quad, row_valid, qpos, window, chunk, keep, lo, scale_log2, m, l, o);
 }
 
 // One head of a token's product (x, D elements, D a multiple of 64) as an MFMA operand: RMSNorm
@@ -1166,7 +1240,7 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
           for (int e = 0; e < 8; ++e) vv[i][e] = (bf16_t)0.0f;
           if (quad == 0) vv[i][0] = vraw[16 * i + r16];
         }
-        tile_update(sc, vv, true, first_pos, quad, row_valid, qpos, a.window, a.chunk, a.scale_log2, m, l, o);
+        tile_update(sc, vv, true, first_pos, quad, row_valid, qpos, a.window, a.chunk, 0, 0, a.scale_log2, m, l, o);
       }
     }
   };
@@ -1193,12 +1267,12 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
     block_pages<P2>(table, min(b + 3 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
     if (FUSED) own_token();  // while the first keys and values are on their way
     while (true) {
-      block_compute(A, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.chunk, a.cap_in, a.cap_out, a.scale_log2, m, l, o);
+      block_compute(A, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.chunk, a.keep_first, a.cap_in, a.cap_out, a.scale_log2, m, l, o);
       block_load<P2, DECODE_ONCE>(a, kvh, min(b + 2 * DW, last) << 5, lo, pos_max, r16, quad, pgA, A, b + 2 * DW <= last);
       block_pages<P2>(table, min(b + 4 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
       b += DW;
       if (b >= b1) break;
-      block_compute(B, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.chunk, a.cap_in, a.cap_out, a.scale_log2, m, l, o);
+      block_compute(B, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.chunk, a.keep_first, a.cap_in, a.cap_out, a.scale_log2, m, l, o);
       block_load<P2, DECODE_ONCE>(a, kvh, min(b + 2 * DW, last) << 5, lo, pos_max, r16, quad, pgB, B, b + 2 * DW <= last);
       block_pages<P2>(table, min(b + 4 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
       b += DW;
@@ -1206,6 +1280,20 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
     }
   } else if (FUSED) {
     own_token();
+  }
+  if (a.keep_first > 0 && split == 0 && wave == 0 && n_rows > 0) {  // uniform over the wave
+    // the kept first keys, all of them before every row's window: one wave walks the few blocks
+    const int kend = min(a.keep_first, lo);
+    if (kend > 0) {
+      if (!FUSED && !(b0 < b1)) {  // no block of the window was this wave's: its queries are still to come
+        const bf16_t* qp = a.q + ((size_t)(q_begin + tok) * a.nq + head) * D;
+#pragma unroll
+        for (int i = 0; i < KFULL; ++i) qreg[i] = *(const bf16x8_t*)(qp + 32 * i + 8 * quad);
+        if (KTAIL) qtail = load_tail(qp + 32 * KFULL, quad);
+      }
+      kept_keys_pass<1, P2>(a, table, kvh, kend, r16, quad, &row_valid, (const bf16x8_t(*)[KFULL > 0 ? KFULL : 1])&qreg, &qtail,
+                            &m, &l, (f32x4_t(*)[DB])&o);
+    }
   }
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -1228,7 +1316,9 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
     float mm = -INFINITY;
 #pragma unroll
     for (int w = 0; w < DW; ++w) mm = fmaxf(mm, lds_m[w * 16 + row]);
-    float num = 0.f, den = 0.f;
+    const bool sink_here = a.sink && a.num_splits == 1;
+    if (sink_here) mm = fmaxf(mm, 0.f);
+    float num = 0.f, den = sink_here ? exp2f(-mm) : 0.f;
     if (mm != -INFINITY) {
 #pragma unroll
       for (int w = 0; w < DW; ++w) {
@@ -1286,6 +1376,7 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
   QRT_CHECK(a.num_splits == 1 || (a.part_o && a.part_lse), "attention: split run without scratch");
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
   QRT_CHECK(a.chunk >= 0 && !(a.chunk > 0 && a.window > 0), "attention: a window or a mask of chunks, not both");
+  QRT_CHECK(a.keep_first >= 0 && (a.keep_first == 0 || a.window > 0), "attention: first keys are kept beside a window");
   QRT_CHECK((a.cap_in > 0.f) == (a.cap_out > 0.f), "attention: a score cap needs both of its factors");
   QRT_CHECK(!a.gate || a.gate_stride >= (long)a.nq * D, "attention: the gate's rows are %ld elements apart, %d heads of %d need more",
             a.gate_stride, a.nq, D);
@@ -1339,7 +1430,7 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
     const int merge_rows = a.merge_tokens ? a.num_merge_tokens * a.nq : num_rows_total;
     if (merge_rows > 0)
       attention_merge_kernel<<<dim3(merge_rows), dim3(D >= 64 ? 64 : 32), 0, stream>>>(
-          a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq, a.gate, a.gate_stride);
+          a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq, a.gate, a.gate_stride, a.sink);
     QRT_LAUNCH_CHECK("attention_merge");
   }
   return 0;
@@ -1356,6 +1447,7 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   QRT_CHECK(a.num_splits == 1 || (a.part_o && a.part_lse), "attention: split run without scratch");
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
   QRT_CHECK(a.chunk >= 0 && !(a.chunk > 0 && a.window > 0), "attention: a window or a mask of chunks, not both");
+  QRT_CHECK(a.keep_first >= 0 && (a.keep_first == 0 || a.window > 0), "attention: first keys are kept beside a window");
   QRT_CHECK((a.cap_in > 0.f) == (a.cap_out > 0.f), "attention: a score cap needs both of its factors");
   QRT_CHECK(!a.gate || a.gate_stride >= (long)a.nq * D, "attention: the gate's rows are %ld elements apart, %d heads of %d need more",
             a.gate_stride, a.nq, D);
@@ -1398,7 +1490,7 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
     const int merge_rows = a.merge_tokens ? a.num_merge_tokens * a.nq : num_rows_total;
     if (merge_rows > 0)
       attention_merge_kernel<<<dim3(merge_rows), dim3(D >= 64 ? 64 : 32), 0, stream>>>(
-          a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq, a.gate, a.gate_stride);
+          a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq, a.gate, a.gate_stride, a.sink);
     QRT_LAUNCH_CHECK("attention_merge");
   }
   return 0;

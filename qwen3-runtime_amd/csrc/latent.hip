@@ -182,6 +182,54 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const T* __restrict__
   }
 }
 
+// Few tokens: one block per (64 outputs of a head), all tokens of the step at once, so that the
+// head's weights are read once a step. Lane j of every wave owns output j of the block's 64 and
+// walks its weight row; the four waves take a quarter of K each, and their partial sums meet in
+// LDS in a fixed order. A token's sum is the same sequence of operations whatever else is in the
+// batch. Tokens go in groups of HL_TOKENS with the inputs in LDS as float32.
+#define HL_TOKENS 8
+template <typename T>
+__global__ __launch_bounds__(256) void heads_linear_rows_kernel(const T* __restrict__ x, long x_row, int in_stride, int in_offset,
+                                                                const T* __restrict__ w, int n, int k, T* __restrict__ out,
+                                                                long out_row, int out_stride, int out_offset, int num_tokens) {
+  extern __shared__ float sm[];
+  float* xs = sm;                        // [HL_TOKENS][k]
+  float* red = sm + HL_TOKENS * k;       // [4][HL_TOKENS][64]
+  const int h = blockIdx.y, j0 = blockIdx.x * 64;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = min(j0 + lane, n - 1);
+  const T* wr = w + ((size_t)h * n + j) * k;
+  const int per = (k + 3) / 4, c0 = min(wave * per, k), c1 = min(k, c0 + per);
+  for (int t0 = 0; t0 < num_tokens; t0 += HL_TOKENS) {
+    const int nt = min(HL_TOKENS, num_tokens - t0);
+    __syncthreads();
+    for (int i = threadIdx.x; i < HL_TOKENS * k; i += 256) {
+      const int t = i / k, c = i - t * k;
+      xs[i] = t < nt ? to_f32<T>(x[(size_t)(t0 + t) * x_row + (size_t)h * in_stride + in_offset + c]) : 0.f;
+    }
+    __syncthreads();
+    float acc[HL_TOKENS];
+#pragma unroll
+    for (int t = 0; t < HL_TOKENS; ++t) acc[t] = 0.f;
+    for (int c = c0; c < c1; ++c) {
+      const float wv = to_f32<T>(wr[c]);
+#pragma unroll
+      for (int t = 0; t < HL_TOKENS; ++t) acc[t] = fmaf(xs[t * k + c], wv, acc[t]);
+    }
+#pragma unroll
+    for (int t = 0; t < HL_TOKENS; ++t) red[(wave * HL_TOKENS + t) * 64 + lane] = acc[t];
+    __syncthreads();
+    for (int i = threadIdx.x; i < nt * 64; i += 256) {
+      const int t = i >> 6, l = i & 63;
+      if (j0 + l < n) {
+        const float sum = ((red[(0 * HL_TOKENS + t) * 64 + l] + red[(1 * HL_TOKENS + t) * 64 + l]) +
+                           red[(2 * HL_TOKENS + t) * 64 + l]) + red[(3 * HL_TOKENS + t) * 64 + l];
+        out[(size_t)(t0 + t) * out_row + (size_t)h * out_stride + out_offset + j0 + l] = from_f32<T>(sum);
+      }
+    }
+  }
+}
+
 extern "C" int qrt_heads_linear(const void* x, long x_row, int in_stride, int in_offset, const void* w, int heads, int n, int k,
                                 void* out, long out_row, int out_stride, int out_offset, int dtype, int num_tokens,
                                 hipStream_t stream) {
@@ -189,6 +237,19 @@ extern "C" int qrt_heads_linear(const void* x, long x_row, int in_stride, int in
   QRT_CHECK(in_offset >= 0 && in_offset + k <= in_stride && (long)heads * in_stride <= x_row && out_offset >= 0 &&
             out_offset + n <= out_stride && (long)heads * out_stride <= out_row, "heads_linear: heads do not fit their rows");
   if (num_tokens == 0) return 0;
+  if (num_tokens <= 64 && k <= 1024) {  // the head's weights once a step
+    const dim3 rows_grid((n + 63) / 64, heads);
+    const size_t rows_lds = (size_t)(HL_TOKENS * k + 4 * HL_TOKENS * 64) * sizeof(float);
+    if (dtype == QRT_F32)
+      heads_linear_rows_kernel<float><<<rows_grid, 256, rows_lds, stream>>>((const float*)x, x_row, in_stride, in_offset, (const float*)w,
+                                                                            n, k, (float*)out, out_row, out_stride, out_offset, num_tokens);
+    else if (dtype == QRT_BF16)
+      heads_linear_rows_kernel<bf16_t><<<rows_grid, 256, rows_lds, stream>>>((const bf16_t*)x, x_row, in_stride, in_offset, (const bf16_t*)w,
+                                                                             n, k, (bf16_t*)out, out_row, out_stride, out_offset, num_tokens);
+    else return qrt_fail("heads_linear: unknown dtype %d", dtype);
+    QRT_LAUNCH_CHECK("heads_linear_rows");
+    return 0;
+  }
   const dim3 grid(num_tokens, heads);
   const size_t lds = (size_t)k * sizeof(float);
   if (dtype == QRT_F32)

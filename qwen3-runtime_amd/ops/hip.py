@@ -81,7 +81,7 @@ class _AttnTileArgs(Structure):
         ("rope", c_void_p), ("slots", c_void_p), ("eps", c_float), ("split_blocks", c_int),
         ("max_items", c_int), ("items", c_void_p),
         ("chunk", c_int), ("cap_in", c_float), ("cap_out", c_float),
-        ("gate", c_void_p), ("gate_stride", c_long),
+        ("gate", c_void_p), ("gate_stride", c_long), ("keep_first", c_int), ("sink", c_int),
     ]
 
 
@@ -1066,15 +1066,15 @@ class HipOps:
         """Whether ``decode_attention`` serves this step: one token per sequence, bfloat16, a head
         size that keeps a rotation pair in one lane (a multiple of 64, up to 256), at most 16
         query heads per key head, and a layer that writes its own cache."""
-        if value_dim not in (None, d) or keep_first or sink:
-            return False  # the kept keys and the sink join in the merge of parts, which reads the queries
+        if value_dim not in (None, d):
+            return False
         return (self.fuse_decode and qkv.dtype == torch.bfloat16 and ctx.max_q_len == 1
                 and ctx.num_tokens == ctx.num_seqs and d % 64 == 0 and d <= 256 and nq // nkv <= 16
                 and cache is not None and cache.writes and cache.group.page_size % 8 == 0
                 and cache.k.dtype == torch.bfloat16)
 
     def decode_attention(self, qkv, cache, ctx, nq, nkv, d, scale, window, q_w, k_w, eps, inv_freq,
-                         angles_key=None, chunk=None, softcap=None, gate=None, value_dim=None):
+                         angles_key=None, chunk=None, softcap=None, gate=None, value_dim=None, keep_first=0, sink=False):
         """``paged_attention(qk_norm_rope_store(qkv, ...))`` for a step of single tokens, in one
         kernel: each block forms its queries from ``qkv`` (RMSNorm per head, NeoX rotation by the
         step's angle table), attends over the cached keys before the token, adds the token's own
@@ -1100,7 +1100,7 @@ class HipOps:
                "rope": None if inv_freq is None else self.rope_table(ctx, inv_freq, angles_key)}
         out = torch.empty((t, nq * d), dtype=qkv.dtype, device=qkv.device)
         self._launch_attention(None, out, cache, ctx, nq, nkv, d, scale, window or 0, None, True, own,
-                               chunk=chunk or 0, softcap=softcap or 0.0, gate=gate)
+                               chunk=chunk or 0, softcap=softcap or 0.0, gate=gate, keep_first=keep_first, sink=sink)
         return out
 
     def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window, chunk=None, softcap=None, value_dim=None,
@@ -1125,8 +1125,9 @@ class HipOps:
         out = torch.empty((t, nq * dv), dtype=q.dtype, device=q.device)
         if keep_first and not window:
             raise OpsError("first keys are kept in sight beside a window")
-        if dv == d and q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0 and not keep_first and not sink:
-            self._attention_mfma(q, out, cache, ctx, nq, nkv, d, scale, window or 0, chunk or 0, softcap or 0.0, gate)
+        if dv == d and q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0:
+            self._attention_mfma(q, out, cache, ctx, nq, nkv, d, scale, window or 0, chunk or 0, softcap or 0.0, gate,
+                                 keep_first=int(keep_first), sink=bool(sink))
         else:
             a = _AttnArgs()
             a.q, a.out, a.k_cache, a.v_cache = q.data_ptr(), out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
@@ -1263,7 +1264,8 @@ class HipOps:
     # mixed steps: sequences with few rows leave the prompt kernel when their context is this long
     split_launch_min_kv = 1024
 
-    def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window, chunk=0, softcap=0.0, gate=None):
+    def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window, chunk=0, softcap=0.0, gate=None,
+                        keep_first=0, sink=False):
         """Which kernel for which sequences. Steps of decoded tokens only: the decode kernel.
         Other steps: the prompt kernels; but sequences of at most 16 rows with a long context
         (decoded tokens beside a prompt portion) would each walk all their keys in one block
@@ -1273,20 +1275,21 @@ class HipOps:
             raise OpsError(f"the bfloat16 attention kernels take a positive score scale, not {scale}")
         g = nq // nkv
         seqs = range(ctx.num_seqs)
+        more = {"keep_first": keep_first, "sink": sink}
         if ctx.max_q_len * g <= 16 and d <= 256:
-            return self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, True, chunk=chunk, softcap=softcap, gate=gate)
+            return self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, True, chunk=chunk, softcap=softcap, gate=gate, **more)
         small = [s for s in seqs if ctx.q_lens_host[s] * g <= 16]
         if (d <= 256 and small and len(small) < ctx.num_seqs
                 and max(ctx.kv_lens_host[s] for s in small) >= self.split_launch_min_kv):
             small_set = set(small)
             big = [s for s in seqs if s not in small_set]
-            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, small, True, chunk=chunk, softcap=softcap, gate=gate)
-            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, big, False, chunk=chunk, softcap=softcap, gate=gate)
+            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, small, True, chunk=chunk, softcap=softcap, gate=gate, **more)
+            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, big, False, chunk=chunk, softcap=softcap, gate=gate, **more)
             return
-        self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, False, chunk=chunk, softcap=softcap, gate=gate)
+        self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, False, chunk=chunk, softcap=softcap, gate=gate, **more)
 
     def _launch_attention(self, q, out, cache, ctx, nq, nkv, d, scale, window, subset, decode, own=None,
-                          chunk=0, softcap=0.0, gate=None):
+                          chunk=0, softcap=0.0, gate=None, keep_first=0, sink=False):
         """One launch over the sequences in ``subset`` (None: all of the step's). ``own``: the
         decode kernel takes the tokens' queries, own keys and own values from the q/k/v product
         (``decode_attention``); ``q`` is then None. ``chunk``: a mask of chunks in place of a
@@ -1336,6 +1339,8 @@ class HipOps:
             self.choose_decode_splits(n_tiles, nkv, seen_kv) if decode else self.choose_splits(n_tiles, nkv, seen_kv))
         a = _AttnTileArgs()
         a.chunk = chunk
+        # beside a window the sequence's first keys stay in sight; a sink: one more term in the softmax's sum
+        a.keep_first, a.sink = int(keep_first), int(bool(sink))
         if softcap:
             a.cap_in, a.cap_out = scale / softcap, softcap / scale
         if gate is not None:

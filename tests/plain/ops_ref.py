@@ -361,14 +361,14 @@ def rotate_half_copy(x, in_stride, in_offset, out, out_stride, out_offset, heads
     ``out[t, h * out_stride + out_offset ...]``, the first ``2 len(freq)`` of them turned: element i
     against element i + len(freq), by ``position * freq[i]`` (float32 angles)."""
     t = x.shape[0]
-    src = x.view(t, heads, in_stride)[:, :, in_offset: in_offset + width].to(torch.float32)
+    src = x[:, : heads * in_stride].reshape(t, heads, in_stride)[:, :, in_offset: in_offset + width].to(torch.float32)
     n = 0 if freq is None else freq.numel()
     if n:
         ang = positions.to(torch.float32)[:, None] * freq.to(torch.float32)[None, :]
         cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
         u, v = src[..., :n], src[..., n: 2 * n]
         src = torch.cat([u * cos - v * sin, v * cos + u * sin, src[..., 2 * n:]], dim=-1)
-    out.view(t, heads, out_stride)[:, :, out_offset: out_offset + width] = src.to(out.dtype)
+    out[:, : heads * out_stride].view(t, heads, out_stride)[:, :, out_offset: out_offset + width] = src.to(out.dtype)
     return out
 
 
