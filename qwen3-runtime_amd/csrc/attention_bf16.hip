@@ -398,7 +398,9 @@ __device__ __forceinline__ void add_sink(float& m, float& l_total, f32x4_t* o) {
 // once into registers and multiplied with all RT tiles, which divides the
 // operand traffic per MFMA by RT.
 template <int RT, bool P2>
-__global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(AttnTileArgs a) {
+// (Heads wider than 256: a wave's accumulator, queries and one block of keys and values fill most of
+// the 512 registers a lane can have, so one block of waves a compute unit and one tile a wave.)
+__global__ __launch_bounds__(256, (RT <= 2 && D <= 256) ? 2 : 1) void attention_bf16_kernel(AttnTileArgs a) {
   const int lane = threadIdx.x & 63, wave = uniform_wave_number();
   const int r16 = lane & 15, quad = lane >> 4;
   // blocks of one tile are neighbours in the launch order, one per key head: with as many key

@@ -40,11 +40,12 @@ __device__ __forceinline__ float row16_sum(float x) {
   return x;
 }
 
-// G groups of four rows a lane: heads of up to 64 G key elements (padded with zero rows)
-template <int G>
+// G groups of four rows a lane: heads of up to 64 G key elements (padded with zero rows). RT_TILE
+// tokens a tile: 16 (8 for the widest heads: what fits 64 KB), or 4 for steps of single tokens,
+// whose blocks then are all resident at once with a quarter of the LDS and of the loads.
+template <int G, int RT_TILE>
 __global__ __launch_bounds__(256) void retention_kernel(RetentionArgs a) {
   constexpr int DP = 64 * G;                          // rows staged
-  constexpr int RT_TILE = G >= 8 ? 8 : 16;            // tokens per LDS tile (the widest heads: what fits 64 KB)
   constexpr int NQK = 2 * RT_TILE * DP / 256;         // q and k elements a thread fetches per tile
   __shared__ __attribute__((aligned(16))) float qs[RT_TILE * DP];
   __shared__ __attribute__((aligned(16))) float ks[RT_TILE * DP];
@@ -163,10 +164,15 @@ extern "C" int qrt_retention(const RetentionArgs* args, int num_tokens, int num_
   if (num_tokens == 0 || num_seqs == 0) return 0;
   const dim3 grid(num_seqs, a.heads, (a.vdim + RT_COLS - 1) / RT_COLS);
   const int groups = (a.dim + 63) / 64;
-  if (groups <= 1) retention_kernel<1><<<grid, 256, 0, stream>>>(a);
-  else if (groups <= 2) retention_kernel<2><<<grid, 256, 0, stream>>>(a);
-  else if (groups <= 4) retention_kernel<4><<<grid, 256, 0, stream>>>(a);
-  else retention_kernel<8><<<grid, 256, 0, stream>>>(a);
+  if (num_tokens <= 2 * num_seqs) {  // decoded tokens, mostly
+    if (groups <= 1) retention_kernel<1, 4><<<grid, 256, 0, stream>>>(a);
+    else if (groups <= 2) retention_kernel<2, 4><<<grid, 256, 0, stream>>>(a);
+    else if (groups <= 4) retention_kernel<4, 4><<<grid, 256, 0, stream>>>(a);
+    else retention_kernel<8, 4><<<grid, 256, 0, stream>>>(a);
+  } else if (groups <= 1) retention_kernel<1, 16><<<grid, 256, 0, stream>>>(a);
+  else if (groups <= 2) retention_kernel<2, 16><<<grid, 256, 0, stream>>>(a);
+  else if (groups <= 4) retention_kernel<4, 16><<<grid, 256, 0, stream>>>(a);
+  else retention_kernel<8, 8><<<grid, 256, 0, stream>>>(a);
   QRT_LAUNCH_CHECK("retention");
   return 0;
 }

@@ -1309,7 +1309,8 @@ class HipOps:
         seen_kv = min(max_kv, reach) if reach else max_kv  # keys that the splits divide
         waves = 1 if max_rows <= 16 else (2 if max_rows <= 32 else 4)
         # long portions: several row tiles per wave, so that loaded keys and values serve more rows
-        row_tiles = 1 if max_rows <= 64 else (self.prefill_row_tiles if d <= 128 else min(2, self.prefill_row_tiles))
+        # (heads wider than 256 fill a lane's registers with one tile)
+        row_tiles = 1 if max_rows <= 64 or d > 256 else (self.prefill_row_tiles if d <= 128 else min(2, self.prefill_row_tiles))
         # the list depends on the rows a tile holds (head geometry and kernel choice): layers of
         # another geometry in the same step get a list of their own
         key = ("attn_plan", g, nkv, d, waves, row_tiles, decode, None if subset is None else tuple(subset), reach)
