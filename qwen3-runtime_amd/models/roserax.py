@@ -126,6 +126,8 @@ def sized(width: int, layers: int, heads: int, kv_heads: int, dim: int, vocab: i
 register_architecture(RoseraxConfig.architecture, RoseraxConfig.from_dict, plan_roserax)
 for _name, _cfg in PRESETS.items():
     register_preset(_name, _cfg.to_dict(), PRESET_PAGE_SIZE.get(_name, 16))
-# layers of the sizes of the 4B dense preset, with a mixture like `deginex_4b_moe`'s in every second
-# layer, for measurements beside it
+# layers of the sizes of the 4B and 8B dense presets, and of a smaller width, with a mixture like
+# `deginex_4b_moe`'s in every second layer, for measurements beside it
 register_preset("roserax_4b", sized(2560, 36, 32, 8, 128, 151936, ff=9728, expert_ff=1536).to_dict(), 16)
+register_preset("roserax_8b", sized(4096, 36, 32, 8, 128, 151936, ff=12288, expert_ff=2048, kv_rank=448, q_rank=1536).to_dict(), 16)
+register_preset("roserax_2b", sized(2048, 28, 16, 4, 128, 151936, ff=6144, expert_ff=1024, kv_rank=256, q_rank=512).to_dict(), 16)
