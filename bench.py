@@ -26,7 +26,9 @@ Other models: ``--preset NAME`` runs the same workload on any registered configu
 designs are measured beside each other at equal sizes: ``--preset deginex_4b`` (hyper-connections,
 chunked capped gated attention, dense feed-forwards) and ``--preset deginex_4b_moe`` (every other
 feed-forward a mixture of 16 experts, 2 a token) have the widths, heads, layers and vocabulary of
-``qwen3_4b``.
+``qwen3_4b``; ``--preset zisedra_4b`` (delta rule beside windowed attention) and ``--preset roserax_4b``
+(latent attention, retention, windowed attention with kept first tokens and a sink) have those sizes
+too, ``*_2b`` and ``*_8b`` smaller and larger ones.
 
 Other workloads: ``--workload mix`` (continuous batching of ``--requests``
 requests with prompts of 128 to 4,096 tokens, portions of 2,048, 256 outputs

@@ -211,10 +211,23 @@ __global__ __launch_bounds__(256) void heads_linear_rows_kernel(const T* __restr
     float acc[HL_TOKENS];
 #pragma unroll
     for (int t = 0; t < HL_TOKENS; ++t) acc[t] = 0.f;
-    for (int c = c0; c < c1; ++c) {
-      const float wv = to_f32<T>(wr[c]);
+    if (sizeof(T) == 2 && (k & 31) == 0 && ((uintptr_t)w & 15) == 0) {
+      // bfloat16 rows whose quarters are whole 16-byte pieces: eight weights a load
+      for (int c = c0; c < c1; c += 8) {
+        const bf16x8_t w8 = *(const bf16x8_t*)((const bf16_t*)wr + c);
 #pragma unroll
-      for (int t = 0; t < HL_TOKENS; ++t) acc[t] = fmaf(xs[t * k + c], wv, acc[t]);
+        for (int e = 0; e < 8; ++e) {
+          const float wv = (float)w8[e];
+#pragma unroll
+          for (int t = 0; t < HL_TOKENS; ++t) acc[t] = fmaf(xs[t * k + c + e], wv, acc[t]);
+        }
+      }
+    } else {
+      for (int c = c0; c < c1; ++c) {
+        const float wv = to_f32<T>(wr[c]);
+#pragma unroll
+        for (int t = 0; t < HL_TOKENS; ++t) acc[t] = fmaf(xs[t * k + c], wv, acc[t]);
+      }
     }
 #pragma unroll
     for (int t = 0; t < HL_TOKENS; ++t) red[(wave * HL_TOKENS + t) * 64 + lane] = acc[t];

@@ -115,7 +115,7 @@ def sized(width: int, layers: int, heads: int, kv_heads: int, dim: int, vocab: i
     and two windowed layers in turn, dense feed-forwards and mixtures alternating."""
     att = WindowSinkSizes(heads, kv_heads, dim, dim, dim ** -0.5, window, keep_first)
     lat = LatentSizes(heads, dim, rot_dim, dim, q_rank, kv_rank, (dim + rot_dim) ** -0.5, _ROT(rot_dim, 1e6))
-    ret = RetentionSizes(heads, dim, dim, tuple(1.0 - 2.0 ** (-5 - 3 * j / max(heads - 1, 1)) for j in range(heads)),
+    ret = RetentionSizes(heads, dim, dim, tuple(1.0 - 0.06 / (1 + j) for j in range(heads)),
                          _ROT(dim, 1e6))
     dense, moe = FeedForwardSizes("dense", ff), FeedForwardSizes("moe", expert_ff, experts=experts, top=top, groups=4, keep=2)
     kinds = (("latent_attention", lat), ("retention", ret), ("attention", att), ("attention", att))

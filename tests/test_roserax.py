@@ -400,7 +400,7 @@ def retention_mixer(width, sizes, eps, w, device, dt):
     (1, 64, 64, (0.99,), 64, 1e4),
     (4, 16, 8, (0.8, 0.8, 0.95, 0.0), 0, 1.0),  # no rotation; a head that remembers only the token itself
     (5, 8, 72, (0.9, 0.91, 0.92, 0.93, 0.94), 2, 10.0),
-    (2, 128, 128, (0.96875, 0.9990234375), 128, 1e6),
+    (2, 128, 128, (0.94, 0.998), 128, 1e6),
     (2, 40, 1, (0.9, 0.99), 20, 100.0),        # one value channel: the read-out's norm leaves its sign
 ])
 def test_retention_against_the_recurrence_written_out(backend, n, d, dv, decay, dims, base):
@@ -680,7 +680,7 @@ def config_g():
     turning elements, experts of 512): the kernel forms that small sizes never reach."""
     return model(500, 1024, [
         {"type": "latent_attention", "mixer": latent(8, 128, 64, 128, 384, 256, 0.07, 1e4), "mlp": dense(2048)},
-        {"type": "retention", "mixer": retention(8, 128, 128, tuple(1 - 2.0 ** (-5 - j / 2) for j in range(8)), 128, 1e4),
+        {"type": "retention", "mixer": retention(8, 128, 128, tuple(1 - 0.08 / (1 + j) for j in range(8)), 128, 1e4),
          "mlp": moe(512, 8, 2, (4, 2))},
         {"type": "attention", "mixer": attention(8, 2, 128, 128, 0.09, 256, 4), "mlp": moe(512, 8, 2, (4, 2))}],
         embedding=4.0), 16
