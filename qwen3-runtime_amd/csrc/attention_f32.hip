@@ -35,7 +35,7 @@ struct AttnArgs {
   int sink;        // 1: one more term exp(0) in the denominator
 };
 
-#define MAX_D 512
+#define MAX_D 1024
 
 template <typename T>
 __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {

@@ -1125,7 +1125,7 @@ class HipOps:
         out = torch.empty((t, nq * dv), dtype=q.dtype, device=q.device)
         if keep_first and not window:
             raise OpsError("first keys are kept in sight beside a window")
-        if dv == d and q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0:
+        if dv == d and q.dtype == torch.bfloat16 and d % 16 == 0 and d <= 512 and ps % 8 == 0:
             self._attention_mfma(q, out, cache, ctx, nq, nkv, d, scale, window or 0, chunk or 0, softcap or 0.0, gate,
                                  keep_first=int(keep_first), sink=bool(sink))
         else:

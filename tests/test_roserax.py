@@ -654,12 +654,13 @@ def config_c():
 
 def config_d():
     """Sizes that are multiples of nothing: width 90, keys of 10, 6 and 14, values of 7, 5 and 3, a
-    window of 13 that keeps none and one of 1 that keeps two, experts of 9, groups of one expert."""
+    window of 13 that keeps none and one of 1 that keeps two, experts of 9, groups of one expert; the
+    last layer has no feed-forward, so the final norm takes the mixer's output through its norm."""
     return model(77, 90, [
         {"type": "attention", "mixer": attention(3, 1, 10, 7, 0.3, 13, 0), "mlp": moe(9, 5, 2, (5, 3))},
         {"type": "latent_attention", "mixer": latent(5, 6, 2, 5, 7, 11, 0.4, 7.0), "mlp": dense(33)},
-        {"type": "retention", "mixer": retention(2, 14, 3, (0.9, 0.95), 6, 50.0), "mlp": None},
-        {"type": "attention", "mixer": attention(2, 2, 6, 6, 0.5, 1, 2), "mlp": dense(20)}], embedding=0.5), 8
+        {"type": "retention", "mixer": retention(2, 14, 3, (0.9, 0.95), 6, 50.0), "mlp": dense(20)},
+        {"type": "attention", "mixer": attention(2, 2, 6, 6, 0.5, 1, 2), "mlp": None}], embedding=0.5), 8
 
 
 def config_e():
