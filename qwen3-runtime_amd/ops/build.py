@@ -19,6 +19,7 @@ import shutil
 import subprocess
 import sys
 import tempfile
+import threading
 import time
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
@@ -80,7 +81,7 @@ def lib_dir() -> Path:
     path = PACKAGE_DIR / "_lib"
     try:
         path.mkdir(exist_ok=True)
-        probe = path / f".probe{os.getpid()}"
+        probe = path / f".probe{os.getpid()}_{threading.get_ident()}"  # builds may run in several threads
         probe.write_text("")
         probe.unlink()
         return path
@@ -177,7 +178,10 @@ def build_library(name: str, force: bool = False) -> Path:
     return so
 
 
-def build_all(head_dims=(16, 32, 48, 64, 80, 96, 112, 128, 256), force: bool = True) -> list[Path]:
-    """Every library the tests, the smoke run and the measurements load."""
+def build_all(head_dims=(16, 32, 48, 64, 80, 96, 112, 128, 160, 176, 256, 320, 448, 512), force: bool = True) -> list[Path]:
+    """Every library the tests, the smoke run and the measurements load (head sizes above 256 are
+    those of latent rows: latent plus turned key part). Three libraries at a time."""
     names = ["core", "peaks"] + [f"attn_bf16_d{d}" for d in head_dims] + registered_libraries()
-    return [build_library(n, force=force) for n in names]
+    first = build_library(names[0], force=force)  # the one with many sources compiles them side by side itself
+    with ThreadPoolExecutor(3) as pool:
+        return [first] + list(pool.map(lambda n: build_library(n, force=force), names[1:]))
