@@ -968,6 +968,7 @@ __device__ __forceinline__ void merge_few(const float* __restrict__ part_o, cons
 }
 
 // out[row] = sum_s 2^(lse_s - M) O_s / sum_s 2^(lse_s - M); empty splits weigh 0
+// (a thread takes two elements of the row: 32, 64 or, for heads wider than 128, 256 threads a row)
 __global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse,
                                        bf16_t* __restrict__ out, int num_splits, const int* __restrict__ tokens,
                                        int nq, const bf16_t* __restrict__ gate, long gate_stride, int sink) {
@@ -1431,7 +1432,7 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
   if (a.num_splits > 1) {
     const int merge_rows = a.merge_tokens ? a.num_merge_tokens * a.nq : num_rows_total;
     if (merge_rows > 0)
-      attention_merge_kernel<<<dim3(merge_rows), dim3(D >= 64 ? 64 : 32), 0, stream>>>(
+      attention_merge_kernel<<<dim3(merge_rows), dim3(D > 128 ? 256 : (D >= 64 ? 64 : 32)), 0, stream>>>(
           a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq, a.gate, a.gate_stride, a.sink);
     QRT_LAUNCH_CHECK("attention_merge");
   }
@@ -1491,7 +1492,7 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   if (a.num_splits > 1) {
     const int merge_rows = a.merge_tokens ? a.num_merge_tokens * a.nq : num_rows_total;
     if (merge_rows > 0)
-      attention_merge_kernel<<<dim3(merge_rows), dim3(D >= 64 ? 64 : 32), 0, stream>>>(
+      attention_merge_kernel<<<dim3(merge_rows), dim3(D > 128 ? 256 : (D >= 64 ? 64 : 32)), 0, stream>>>(
           a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq, a.gate, a.gate_stride, a.sink);
     QRT_LAUNCH_CHECK("attention_merge");
   }

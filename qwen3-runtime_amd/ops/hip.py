@@ -1205,9 +1205,13 @@ class HipOps:
     key_groups_ratio = 0.9
 
     @staticmethod
-    def choose_splits(num_tiles: int, nkv: int, max_kv: int) -> int:
-        """Portions: how many ways to split the keys so that few long sequences still fill the chip."""
+    def choose_splits(num_tiles: int, nkv: int, max_kv: int, head_dim: int = 0) -> int:
+        """Portions: how many ways to split the keys so that few long sequences still fill the chip.
+        Heads wider than 256 (one block of waves a compute unit, and no decode kernel of their own, so
+        that decoded tokens come here too): parts of 64 keys and more, 256 blocks in all."""
         work = num_tiles * nkv
+        if head_dim > 256:
+            return 1 if max_kv <= 128 or work >= 256 else max(1, min((max_kv + 63) // 64, (256 + work - 1) // work, 64))
         if max_kv <= 512 or work >= 512:
             return 1
         return max(1, min((max_kv + 255) // 256, (1024 + work - 1) // work, 64))
@@ -1337,7 +1341,7 @@ class HipOps:
             ctx.scratch[key] = plan
         tiles, n_tiles, tokens, groups = plan
         splits = ctx.scratch.get("attn_splits") or (
-            self.choose_decode_splits(n_tiles, nkv, seen_kv) if decode else self.choose_splits(n_tiles, nkv, seen_kv))
+            self.choose_decode_splits(n_tiles, nkv, seen_kv) if decode else self.choose_splits(n_tiles, nkv, seen_kv, d))
         a = _AttnTileArgs()
         a.chunk = chunk
         # beside a window the sequence's first keys stay in sight; a sink: one more term in the softmax's sum
