@@ -183,6 +183,9 @@ def window_mixer(width, sizes, eps, w, device, dt):
     (2, 1, 128, 128, 130, 0, 16),  # none kept
     (5, 5, 8, 8, 1, 3, 8),         # a window of the query itself
     (8, 2, 96, 96, 33, 7, 32),
+    (4, 2, 32, 32, 40, 70, 16),    # kept tokens over three blocks of 32 keys
+    (2, 1, 64, 64, 24, 64, 16),    # ... exactly two
+    (4, 4, 128, 128, 50, 33, 16),
 ])
 def test_window_keeps_first_tokens_and_has_a_sink(backend, heads, kv_heads, d, dv, window, keep, page):
     """The attention mixer (normed queries and keys, no rotation, window, kept first tokens, sink) over
@@ -677,13 +680,13 @@ def config_e():
 
 
 def config_g():
-    """Layers of a real model's proportions (heads of 128, a window of 256, a latent of 256 with 64
+    """Layers of a real model's proportions (heads of 128, a window of 256 that keeps 40 tokens, a latent of 256 with 64
     turning elements, experts of 512): the kernel forms that small sizes never reach."""
     return model(500, 1024, [
         {"type": "latent_attention", "mixer": latent(8, 128, 64, 128, 384, 256, 0.07, 1e4), "mlp": dense(2048)},
         {"type": "retention", "mixer": retention(8, 128, 128, tuple(1 - 0.08 / (1 + j) for j in range(8)), 128, 1e4),
          "mlp": moe(512, 8, 2, (4, 2))},
-        {"type": "attention", "mixer": attention(8, 2, 128, 128, 0.09, 256, 4), "mlp": moe(512, 8, 2, (4, 2))}],
+        {"type": "attention", "mixer": attention(8, 2, 128, 128, 0.09, 256, 40), "mlp": moe(512, 8, 2, (4, 2))}],
         embedding=4.0), 16
 
 
