@@ -854,6 +854,25 @@ def test_long_decoding_in_a_pool_of_one_window(folder, backend):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
+def test_decoded_tokens_over_a_long_context_beside_prompt_portions(folder, backend):
+    """One request decodes past 1,000 tokens while another is read in portions in the same steps: the
+    attention of the few rows with the long context is cut over many blocks in a launch of its own,
+    whose parts a merge joins (with the sink, after the kept first keys), beside the portions'."""
+    raw, page = config_e()
+    reqs = traces.make_requests(raw["vocab"], [1085, 700], seed=11)
+    a, b = reqs["r0"], reqs["r1"]
+    steps = [{"step": 0, "entries": [{"id": "r0", "tokens": a[:1060], "want": [0, 500, 1059]}], "end": []}]
+    for i in range(25):
+        steps.append({"step": i + 1, "end": ["r0", "r1"] if i == 24 else [], "entries": [
+            {"id": "r0", "tokens": a[1060 + i: 1061 + i], "want": [0]},
+            {"id": "r1", "tokens": b[28 * i: 28 * (i + 1)], "want": [0, 27]}]})
+    loaded = load(folder("e", backend[1]), page, traces.peak_tokens(steps, unit=page) // page, backend)
+    got = traces.replay(loaded, steps, poison_freed=True)
+    want = plain_logits(folder("e", backend[1]), reqs)
+    check(got, {k: want[k] for k in got}, backend[1], NOISE["e"])
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
 def test_batch_mates_do_not_change_a_request(folder, backend):
     """Unequal requests in one batch against each alone: the same logits within rounding."""
     raw, page = config_a()
