@@ -237,6 +237,100 @@ extern "C" int qrt_norm_add_rmsnorm(float* residual, const void* y, int y_code, 
   return 0;
 }
 
+// ------------------------------------------------ a sum of scaled sub-layer outputs, then the norm
+// x = residual[r] + sum_i s_i * y_i[r]  (element by element; written back without `rows`);
+// out[b] = x / rms(x) * w.  Everything float32. One block of 1,024 threads per row; a thread keeps
+// its elements in registers (rows up to 4,096 wide; the rest of a wider row is computed again),
+// all terms, vectors and weights asked for before the first is used. The terms are added in order.
+#define SA_TERMS 4
+struct ScaledTerms {
+  Planes y[SA_TERMS];
+  const float* scale[SA_TERMS];
+  int count;
+};
+
+__device__ __forceinline__ float scaled_sum_at(const ScaledTerms& s, float x, size_t at, int i) {
+  float part[SA_TERMS], sc[SA_TERMS];
+#pragma unroll
+  for (int k = 0; k < SA_TERMS; ++k) {
+    const int kk = k < s.count ? k : 0;
+    part[k] = planes_at(s.y[kk], at);
+    sc[k] = s.scale[kk][i];
+  }
+#pragma unroll
+  for (int k = 0; k < SA_TERMS; ++k)
+    if (k < s.count) x = fmaf(sc[k], part[k], x);
+  return x;
+}
+
+template <typename TO>
+__global__ __launch_bounds__(1024) void scaled_add_rmsnorm_kernel(float* __restrict__ residual, ScaledTerms s,
+                                                                  const float* __restrict__ weight, float eps,
+                                                                  const int* __restrict__ rows, TO* __restrict__ out,
+                                                                  int hidden) {
+  __shared__ float red[32];
+  const int b = blockIdx.x;
+  const int r = rows ? rows[b] : b;
+  const size_t row = (size_t)r * hidden;
+  float vx[NM_KEEP], wn[NM_KEEP];
+#pragma unroll
+  for (int j = 0; j < NM_KEEP; ++j) {
+    const int i = min((int)threadIdx.x + 1024 * j, hidden - 1);
+    vx[j] = scaled_sum_at(s, residual[row + i], row + i, i);
+    wn[j] = weight[i];
+  }
+  float sx = 0.f;
+#pragma unroll
+  for (int j = 0; j < NM_KEEP; ++j) {
+    const int i = threadIdx.x + 1024 * j;
+    if (i < hidden) {
+      sx += vx[j] * vx[j];
+      if (!rows) residual[row + i] = vx[j];
+    }
+  }
+  for (int i = threadIdx.x + 1024 * NM_KEEP; i < hidden; i += 1024) {
+    const float x = scaled_sum_at(s, residual[row + i], row + i, i);
+    sx += x * x;
+    if (!rows) residual[row + i] = x;
+  }
+  sx = block_sum(sx, red);
+  const float ix = 1.0f / sqrtf(sx / (float)hidden + eps);
+#pragma unroll
+  for (int j = 0; j < NM_KEEP; ++j) {
+    const int i = threadIdx.x + 1024 * j;
+    if (i < hidden) out[(size_t)b * hidden + i] = from_f32<TO>(vx[j] * ix * wn[j]);
+  }
+  for (int i = threadIdx.x + 1024 * NM_KEEP; i < hidden; i += 1024) {
+    const float x = rows ? scaled_sum_at(s, residual[row + i], row + i, i) : residual[row + i];
+    out[(size_t)b * hidden + i] = from_f32<TO>(x * ix * weight[i]);
+  }
+}
+
+// y, y_code, y_planes, scale: `count` entries each; all planes [P, T, H] lie `plane_stride` elements apart
+extern "C" int qrt_scaled_add_rmsnorm(float* residual, const void* const* y, const int* y_code, const int* y_planes,
+                                      const float* const* scale, int count, long plane_stride, const float* weight,
+                                      float eps, const int* rows, void* out, int out_dtype, int num_out, int hidden,
+                                      hipStream_t stream) {
+  QRT_CHECK(num_out >= 0 && hidden > 0 && count >= 1 && count <= SA_TERMS, "scaled_add_rmsnorm: %d terms (1..%d)", count, SA_TERMS);
+  ScaledTerms s;
+  s.count = count;
+  for (int k = 0; k < SA_TERMS; ++k) {
+    const int kk = k < count ? k : 0;
+    QRT_CHECK(y[kk] && scale[kk] && y_planes[kk] >= 1, "scaled_add_rmsnorm: term %d is not there", kk);
+    QRT_CHECK(y_code[kk] == QRT_F32 || (y_code[kk] == QRT_BF16 && y_planes[kk] == 1), "scaled_add_rmsnorm: planes are float32");
+    s.y[k] = Planes{y[kk], y_code[kk], y_planes[kk], plane_stride};
+    s.scale[k] = scale[kk];
+  }
+  if (num_out == 0) return 0;
+  if (out_dtype == QRT_F32)
+    scaled_add_rmsnorm_kernel<float><<<num_out, 1024, 0, stream>>>(residual, s, weight, eps, rows, (float*)out, hidden);
+  else if (out_dtype == QRT_BF16)
+    scaled_add_rmsnorm_kernel<bf16_t><<<num_out, 1024, 0, stream>>>(residual, s, weight, eps, rows, (bf16_t*)out, hidden);
+  else return qrt_fail("scaled_add_rmsnorm: unknown dtype %d", out_dtype);
+  QRT_LAUNCH_CHECK("scaled_add_rmsnorm");
+  return 0;
+}
+
 // ------------------------------------------------ small elementwise steps
 // x *= factor, float32, in place (logits times a constant)
 __global__ void scale_kernel(float* __restrict__ x, float factor, long n) {

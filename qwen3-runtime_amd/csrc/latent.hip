@@ -7,11 +7,28 @@
 //   key/value head is [c | k_rot], its value row [c | 0] (keys [page, 1, offset, W], values
 //   [page, 1, W, offset], W = rank + rot_dim);
 // * a copy of `width` elements per (token, head) from one strided layout to another with the
-//   first 2 n of them turned, element i against element i + n, by position * freq[i] (the
-//   "rotate half" layout; angles, sines and cosines float32);
+//   first 2 n of them turned, element i against element i + n (the "rotate half" layout), or,
+//   with `neighbours`, element 2i against element 2i + 1, by position * freq[i] (angles, sines
+//   and cosines float32; sines and cosines times `magnitude`); the cached row's rotated part
+//   takes the same two options;
 // * a product per head, out[t, h, :] = W[h] x[t, h, :], on strided rows: W [heads, N, K].
 #include "common.h"
 #include <math.h>
+
+// Element i of a vector whose first 2 `pairs` elements turn: its partner and the pair's number.
+// Half layout: i against i + pairs; neighbours: 2j against 2j + 1. `first` says whether i is the
+// pair's first element (x cos - other sin) or its second (x cos + other sin).
+__device__ __forceinline__ void rotation_partner(int i, int pairs, int neighbours, int* pair, int* other, bool* first) {
+  if (neighbours) {
+    *pair = i >> 1;
+    *first = (i & 1) == 0;
+    *other = i ^ 1;
+  } else {
+    *first = i < pairs;
+    *pair = *first ? i : i - pairs;
+    *other = *first ? i + pairs : i - pairs;
+  }
+}
 
 // ---------------------------------------------------------------- norm of some columns
 template <typename T>
@@ -50,7 +67,8 @@ __global__ __launch_bounds__(256) void latent_store_kernel(const T* __restrict__
                                                            int rot_dim, const float* __restrict__ weight, float eps,
                                                            const int* __restrict__ positions, const float* __restrict__ freq,
                                                            int pairs, const int* __restrict__ slots, T* __restrict__ k_cache,
-                                                           T* __restrict__ v_cache, int page_size) {
+                                                           T* __restrict__ v_cache, int page_size, int neighbours,
+                                                           float magnitude) {
   __shared__ float red[32];
   const int t = blockIdx.x;
   const T* row = y + (size_t)t * stride + first;
@@ -76,11 +94,15 @@ __global__ __launch_bounds__(256) void latent_store_kernel(const T* __restrict__
   for (int i = threadIdx.x; i < rot_dim; i += 256) {
     float x = to_f32<T>(rot[i]);
     if (i < 2 * pairs) {
-      const int j = i < pairs ? i : i - pairs;
+      int j, o;
+      bool first;
+      rotation_partner(i, pairs, neighbours, &j, &o, &first);
       float sn, cs;
       sincos_angle(pos * freq[j], &sn, &cs);
-      const float other = to_f32<T>(rot[i < pairs ? i + pairs : i - pairs]);
-      x = i < pairs ? x * cs - other * sn : x * cs + other * sn;
+      sn *= magnitude;
+      cs *= magnitude;
+      const float other = to_f32<T>(rot[o]);
+      x = first ? x * cs - other * sn : x * cs + other * sn;
     }
     kr[rank + i] = from_f32<T>(x);
     vr[(size_t)(rank + i) * page_size] = from_f32<T>(0.f);
@@ -89,7 +111,8 @@ __global__ __launch_bounds__(256) void latent_store_kernel(const T* __restrict__
 
 extern "C" int qrt_latent_store(const void* y, long stride, int first, int rank, int rot_dim, const float* weight, float eps,
                                 const int* positions, const float* freq, int pairs, const int* slots, void* k_cache,
-                                void* v_cache, int page_size, long num_pages, int dtype, int num_tokens, hipStream_t stream) {
+                                void* v_cache, int page_size, long num_pages, int dtype, int num_tokens, int neighbours,
+                                float magnitude, hipStream_t stream) {
   QRT_CHECK(num_tokens >= 0 && rank > 0 && rot_dim >= 0 && first >= 0 && (long)first + rank + rot_dim <= stride,
             "latent_store: bad sizes");
   QRT_CHECK(pairs >= 0 && 2 * pairs <= rot_dim && (pairs == 0 || freq), "latent_store: %d pairs in %d elements", pairs, rot_dim);
@@ -97,10 +120,10 @@ extern "C" int qrt_latent_store(const void* y, long stride, int first, int rank,
   if (num_tokens == 0) return 0;
   if (dtype == QRT_F32)
     latent_store_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)y, stride, first, rank, rot_dim, weight, eps, positions,
-                                                               freq, pairs, slots, (float*)k_cache, (float*)v_cache, page_size);
+                                                               freq, pairs, slots, (float*)k_cache, (float*)v_cache, page_size, neighbours, magnitude);
   else if (dtype == QRT_BF16)
     latent_store_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)y, stride, first, rank, rot_dim, weight, eps, positions,
-                                                                freq, pairs, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size);
+                                                                freq, pairs, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size, neighbours, magnitude);
   else return qrt_fail("latent_store: unknown dtype %d", dtype);
   QRT_LAUNCH_CHECK("latent_store");
   return 0;
@@ -113,6 +136,7 @@ struct RotateArgs {
   int heads, width, pairs;
   const int* positions; const float* freq;
   int scale_from_head; float scale;  // heads from this one on are multiplied by `scale` after turning
+  int neighbours; float magnitude;   // pairs of neighbours instead of halves; what multiplies sines and cosines
 };
 
 template <typename TI, typename TO>
@@ -127,11 +151,15 @@ __global__ __launch_bounds__(256) void rotate_half_kernel(RotateArgs a) {
     const TI* src = xr + (size_t)h * a.in_stride;
     float x = to_f32<TI>(src[i]);
     if (i < 2 * a.pairs) {
-      const int j = i < a.pairs ? i : i - a.pairs;
+      int j, o;
+      bool first;
+      rotation_partner(i, a.pairs, a.neighbours, &j, &o, &first);
       float sn, cs;
       sincos_angle(pos * a.freq[j], &sn, &cs);
-      const float other = to_f32<TI>(src[i < a.pairs ? i + a.pairs : i - a.pairs]);
-      x = i < a.pairs ? x * cs - other * sn : x * cs + other * sn;
+      sn *= a.magnitude;
+      cs *= a.magnitude;
+      const float other = to_f32<TI>(src[o]);
+      x = first ? x * cs - other * sn : x * cs + other * sn;
     }
     if (h >= a.scale_from_head) x *= a.scale;
     orow[(size_t)h * a.out_stride + i] = from_f32<TO>(x);

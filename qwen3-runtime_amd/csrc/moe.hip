@@ -4,7 +4,9 @@
 // Router: logits z[e] = x . W_r[e] + b[e] in float32 (the router's matrix is held in float32
 // in every mode), the `top` largest per token (ties: the lower index), softmax over those; or,
 // with sigmoid scores, the `top` largest sigmoid(z), which weigh the experts as they are; or, with
-// softmax scores over all experts (`sigmoid_scores` = 2), the `top` largest of those, likewise. Experts
+// softmax scores over all experts (`sigmoid_scores` = 2), the `top` largest of those, likewise. With
+// scores, a `correction` per expert may be added for the choice alone, the chosen scores may be
+// divided by their sum (+ 1e-20, `renormalise`), and the weights are multiplied by `weight_scale`. Experts
 // may form equal groups of neighbours of which only the `keep` best (by the sum of a group's two
 // largest entries, or with `group_max` by its largest) stay in the choice.
 // Experts: pair p = (token t, its j-th expert e) computes act[p] = silu(G_e x) * (U_e x) (or the
@@ -35,6 +37,17 @@ __device__ __forceinline__ float lane_dot(const T* __restrict__ w, const float* 
   return acc;
 }
 
+// An expert's activation: the gated ones of common.h, or, for experts without a gate, the square
+// of relu of the one product (`u` unused).
+#define QRT_ACT_RELU2 2
+__device__ __forceinline__ float expert_act(float g, float u, int kind, float limit) {
+  if (kind == QRT_ACT_RELU2) {
+    g = fmaxf(g, 0.f);
+    return g * g;
+  }
+  return gated_act(g, u, kind, limit);
+}
+
 // ------------------------------------------------------------------- router
 #define MAX_EXPERTS 1024
 // One block of 16 waves per token. A wave takes the experts wave, wave + 16, ...: its lanes read
@@ -44,7 +57,9 @@ template <typename T>
 __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x, const float* __restrict__ router,
                                                          const float* __restrict__ bias, int* __restrict__ index,
                                                          float* __restrict__ weight, int hidden, int experts, int top,
-                                                         int sigmoid_scores, int groups, int keep, int group_max) {
+                                                         int sigmoid_scores, int groups, int keep, int group_max,
+                                                         const float* __restrict__ correction, int renormalise,
+                                                         float weight_scale) {
   __shared__ float logit[MAX_EXPERTS];
   __shared__ float score[MAX_EXPERTS];
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -81,6 +96,11 @@ __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x
     for (int e = 0; e < experts; ++e) sum += expf(logit[e] - mx);
     __builtin_amdgcn_wave_barrier();
     for (int e = lane; e < experts; e += 64) score[e] = logit[e] = expf(logit[e] - mx) / sum;
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (correction) {
+    // the choice goes by score + correction; the weights stay the scores
+    for (int e = lane; e < experts; e += 64) logit[e] += correction[e];
     __builtin_amdgcn_wave_barrier();
   }
   if (groups > 1 && keep < groups) {
@@ -139,24 +159,31 @@ __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x
     }
     __builtin_amdgcn_wave_barrier();
   }
-  if (lane < top) weight[(size_t)t * top + lane] = sigmoid_scores ? chosen : chosen / denom;
+  if (lane < top) {
+    float w = sigmoid_scores ? chosen : chosen / denom;
+    if (renormalise) w = w / (denom + 1e-20f);  // denom: the chosen scores' sum, in the order of the choice
+    weight[(size_t)t * top + lane] = w * weight_scale;
+  }
 }
 
 extern "C" int qrt_route_top(const void* x, int x_dtype, const float* router, const float* bias, int* index,
                              float* weight, int num_tokens, int hidden, int experts, int top, int sigmoid_scores,
-                             int groups, int keep, int group_max, hipStream_t stream) {
+                             int groups, int keep, int group_max, const float* correction, int renormalise,
+                             float weight_scale, hipStream_t stream) {
   QRT_CHECK(groups >= 1 && groups <= 64 && experts % groups == 0 && keep >= 1 && keep <= groups &&
             (long)keep * (experts / groups) >= top,
             "route_top: %d groups of which %d stay do not fit %d experts of which %d are chosen", groups, keep, experts, top);
   QRT_CHECK(num_tokens >= 0 && hidden > 0, "route_top: bad sizes T=%d H=%d", num_tokens, hidden);
+  QRT_CHECK(sigmoid_scores != 0 || (!correction && !renormalise),
+            "route_top: a correction of the choice and renormalised weights go with scores over all experts");
   QRT_CHECK(experts >= 1 && experts <= MAX_EXPERTS && top >= 1 && top <= experts && top <= 64,
             "route_top: %d of %d experts (at most %d experts, 64 chosen)", top, experts, MAX_EXPERTS);
   if (num_tokens == 0) return 0;
   dim3 grid(num_tokens), block(1024);
   if (x_dtype == QRT_F32)
-    route_top_kernel<float><<<grid, block, 0, stream>>>((const float*)x, router, bias, index, weight, hidden, experts, top, sigmoid_scores, groups, keep, group_max);
+    route_top_kernel<float><<<grid, block, 0, stream>>>((const float*)x, router, bias, index, weight, hidden, experts, top, sigmoid_scores, groups, keep, group_max, correction, renormalise, weight_scale);
   else if (x_dtype == QRT_BF16)
-    route_top_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, router, bias, index, weight, hidden, experts, top, sigmoid_scores, groups, keep, group_max);
+    route_top_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, router, bias, index, weight, hidden, experts, top, sigmoid_scores, groups, keep, group_max, correction, renormalise, weight_scale);
   else return qrt_fail("route_top: unknown dtype %d", x_dtype);
   QRT_LAUNCH_CHECK("route_top");
   return 0;
@@ -175,15 +202,16 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
   for (int c = threadIdx.x; c < hidden; c += 256) xs[c] = to_f32<T>(x[(size_t)t * hidden + c]);
   __syncthreads();
   const bool wide = hidden % (16 / sizeof(T)) == 0;
-  const T* w = gate_up + (size_t)e * 2 * inter * hidden;
+  const bool gated = act_kind != QRT_ACT_RELU2;  // without a gate an expert's rows are the up rows alone
+  const T* w = gate_up + (size_t)e * (gated ? 2 : 1) * inter * hidden;
   const int i0 = (blockIdx.y * 4 + wave) * ROWS_PER_WAVE;
 #pragma unroll
   for (int r = 0; r < ROWS_PER_WAVE; ++r) {
     const int i = i0 + r;
     if (i >= inter) break;
     const float g = wave_sum(lane_dot<T>(w + (size_t)i * hidden, xs, hidden, lane, wide));
-    const float u = wave_sum(lane_dot<T>(w + (size_t)(inter + i) * hidden, xs, hidden, lane, wide));
-    if (lane == 0) act[(size_t)p * inter + i] = from_f32<T>(gated_act(g, u, act_kind, limit));
+    const float u = gated ? wave_sum(lane_dot<T>(w + (size_t)(inter + i) * hidden, xs, hidden, lane, wide)) : 0.f;
+    if (lane == 0) act[(size_t)p * inter + i] = from_f32<T>(expert_act(g, u, act_kind, limit));
   }
 }
 
@@ -216,7 +244,7 @@ extern "C" int qrt_moe_pairs(const void* x, const void* gate_up, const void* dow
                              const float* weight, void* act, float* out, int dtype, int num_tokens, int hidden,
                              int inter, int experts, int top, int act_kind, float limit, hipStream_t stream) {
   QRT_CHECK(num_tokens >= 0 && hidden > 0 && inter > 0 && experts > 0 && top > 0, "moe: bad sizes");
-  QRT_CHECK(act_kind == QRT_ACT_SWIGLU || act_kind == QRT_ACT_CLAMPED, "moe: unknown activation %d", act_kind);
+  QRT_CHECK(act_kind == QRT_ACT_SWIGLU || act_kind == QRT_ACT_CLAMPED || act_kind == QRT_ACT_RELU2, "moe: unknown activation %d", act_kind);
   QRT_CHECK((size_t)hidden * 4 <= 64 * 1024 && (size_t)top * inter * 4 <= 64 * 1024,
             "moe: a token's row (%d) or its experts' inner rows (%d x %d) do not fit", hidden, top, inter);
   QRT_CHECK(dtype == QRT_F32 || dtype == QRT_BF16, "moe: unknown dtype %d", dtype);
@@ -339,17 +367,20 @@ extern "C" int qrt_moe_combine(const void* y, const int* place, const int* index
 // owns a few rows of one expert's matrix: it brings them into LDS once and multiplies them
 // with every token of that expert, a token per wave at a time, the token's row read from
 // memory in 16-byte pieces. Blocks of experts that nobody chose leave at once. No count ever
-// reaches the host, so the form can be captured into a graph. GATED: the rows are R gate rows
-// and the R up rows that go with them, the input is the tokens' matrix and the output
-// silu(gate) * up by pair; otherwise R rows of the down matrix, the input by pair and the
+// reaches the host, so the form can be captured into a graph. MODE 1 (gated): the rows are R gate
+// rows and the R up rows that go with them, the input is the tokens' matrix and the output
+// silu(gate) * up by pair; MODE 2: R up rows of experts without a gate, the output their
+// activation by pair; MODE 0: R rows of the down matrix, the input by pair and the
 // output by place (moe_combine weighs and sums it). Every output element is one wave's sum in a
 // fixed order.
-template <typename T, int R, bool GATED>
+template <typename T, int R, int MODE>
 __global__ __launch_bounds__(256) void moe_rows_by_expert_kernel(const T* __restrict__ in, const T* __restrict__ w,
                                                                  const int* __restrict__ order,
                                                                  const int* __restrict__ offsets, T* __restrict__ out,
                                                                  int K, int N, int top, int act_kind, float limit) {
   constexpr int VEC = 16 / sizeof(T);
+  constexpr bool GATED = MODE == 1;
+  constexpr bool FIRST = MODE != 0;  // the experts' first product: input by token, output by pair
   constexpr int NR = GATED ? 2 * R : R;
   typedef T vec_t __attribute__((ext_vector_type(VEC)));
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -374,7 +405,7 @@ __global__ __launch_bounds__(256) void moe_rows_by_expert_kernel(const T* __rest
   __syncthreads();
   for (int i = wave; i < count; i += 4) {
     const int p = order[first + i];
-    const T* xr = in + (size_t)(GATED ? p / top : p) * K;
+    const T* xr = in + (size_t)(FIRST ? p / top : p) * K;
     float acc[NR];
 #pragma unroll
     for (int r = 0; r < NR; ++r) acc[r] = 0.f;
@@ -397,31 +428,31 @@ __global__ __launch_bounds__(256) void moe_rows_by_expert_kernel(const T* __rest
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if (n0 + r >= N) break;
-        if (GATED) out[(size_t)p * N + n0 + r] = from_f32<T>(gated_act(acc[r], acc[R + r], act_kind, limit));
+        if (FIRST) out[(size_t)p * N + n0 + r] = from_f32<T>(expert_act(acc[r], GATED ? acc[NR - R + r] : 0.f, act_kind, limit));
         else out[(size_t)(first + i) * N + n0 + r] = from_f32<T>(acc[r]);
       }
     }
   }
 }
 
-template <typename T, int R, bool GATED>
+template <typename T, int R, int MODE>
 static void moe_rows_launch(const void* in, const void* w, const int* order, const int* offsets, void* out, int K, int N,
                             int experts, int top, int act_kind, float limit, hipStream_t stream) {
   dim3 grid(experts, (N + R - 1) / R);
-  const size_t smem = (size_t)(GATED ? 2 * R : R) * K * sizeof(T);
-  moe_rows_by_expert_kernel<T, R, GATED><<<grid, 256, smem, stream>>>((const T*)in, (const T*)w, order, offsets, (T*)out, K, N, top, act_kind, limit);
+  const size_t smem = (size_t)(MODE == 1 ? 2 * R : R) * K * sizeof(T);
+  moe_rows_by_expert_kernel<T, R, MODE><<<grid, 256, smem, stream>>>((const T*)in, (const T*)w, order, offsets, (T*)out, K, N, top, act_kind, limit);
 }
 
-template <typename T, bool GATED>
+template <typename T, int MODE>
 static int moe_rows_pick(const void* in, const void* w, const int* order, const int* offsets, void* out, int K, int N,
                          int experts, int top, int act_kind, float limit, hipStream_t stream) {
   // as many rows a block as 48 KB of LDS hold, eight at most
-  const size_t row_bytes = (size_t)(GATED ? 2 : 1) * K * sizeof(T);
+  const size_t row_bytes = (size_t)(MODE == 1 ? 2 : 1) * K * sizeof(T);
   const int fit = (int)(48 * 1024 / row_bytes);
-  if (fit >= 8) moe_rows_launch<T, 8, GATED>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
-  else if (fit >= 4) moe_rows_launch<T, 4, GATED>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
-  else if (fit >= 2) moe_rows_launch<T, 2, GATED>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
-  else if (fit >= 1) moe_rows_launch<T, 1, GATED>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
+  if (fit >= 8) moe_rows_launch<T, 8, MODE>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
+  else if (fit >= 4) moe_rows_launch<T, 4, MODE>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
+  else if (fit >= 2) moe_rows_launch<T, 2, MODE>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
+  else if (fit >= 1) moe_rows_launch<T, 1, MODE>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
   else return qrt_fail("moe: rows of %d elements do not fit the block's memory", K);
   return 0;
 }
@@ -431,18 +462,22 @@ extern "C" int qrt_moe_by_expert(const void* x, const void* gate_up, const void*
                                  const int* offsets, void* act, void* y, int dtype, int hidden, int inter, int experts,
                                  int top, int act_kind, float limit, hipStream_t stream) {
   QRT_CHECK(hidden > 0 && inter > 0 && experts >= 1 && experts <= MAX_EXPERTS && top > 0, "moe: bad sizes");
-  QRT_CHECK(act_kind == QRT_ACT_SWIGLU || act_kind == QRT_ACT_CLAMPED, "moe: unknown activation %d", act_kind);
+  QRT_CHECK(act_kind == QRT_ACT_SWIGLU || act_kind == QRT_ACT_CLAMPED || act_kind == QRT_ACT_RELU2, "moe: unknown activation %d", act_kind);
   QRT_CHECK(dtype == QRT_F32 || dtype == QRT_BF16, "moe: unknown dtype %d", dtype);
   const int vec = dtype == QRT_F32 ? 4 : 8;
   QRT_CHECK(hidden % vec == 0 && inter % vec == 0, "moe: widths %d and %d are no multiples of %d", hidden, inter, vec);
   QRT_CHECK((inter + 0) / 1 <= 65535 * 8 && hidden <= 65535 * 8, "moe: rows too many for one launch");
   int rc;
   if (dtype == QRT_F32) {
-    rc = moe_rows_pick<float, true>(x, gate_up, order, offsets, act, hidden, inter, experts, top, act_kind, limit, stream);
-    if (rc == 0) rc = moe_rows_pick<float, false>(act, down, order, offsets, y, inter, hidden, experts, top, act_kind, limit, stream);
+    rc = act_kind == QRT_ACT_RELU2
+             ? moe_rows_pick<float, 2>(x, gate_up, order, offsets, act, hidden, inter, experts, top, act_kind, limit, stream)
+             : moe_rows_pick<float, 1>(x, gate_up, order, offsets, act, hidden, inter, experts, top, act_kind, limit, stream);
+    if (rc == 0) rc = moe_rows_pick<float, 0>(act, down, order, offsets, y, inter, hidden, experts, top, act_kind, limit, stream);
   } else {
-    rc = moe_rows_pick<bf16_t, true>(x, gate_up, order, offsets, act, hidden, inter, experts, top, act_kind, limit, stream);
-    if (rc == 0) rc = moe_rows_pick<bf16_t, false>(act, down, order, offsets, y, inter, hidden, experts, top, act_kind, limit, stream);
+    rc = act_kind == QRT_ACT_RELU2
+             ? moe_rows_pick<bf16_t, 2>(x, gate_up, order, offsets, act, hidden, inter, experts, top, act_kind, limit, stream)
+             : moe_rows_pick<bf16_t, 1>(x, gate_up, order, offsets, act, hidden, inter, experts, top, act_kind, limit, stream);
+    if (rc == 0) rc = moe_rows_pick<bf16_t, 0>(act, down, order, offsets, y, inter, hidden, experts, top, act_kind, limit, stream);
   }
   if (rc != 0) return rc;
   QRT_LAUNCH_CHECK("moe_by_expert");

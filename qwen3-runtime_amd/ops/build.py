@@ -35,7 +35,7 @@ FLAGS = [
 # further hipcc flags (for instance -D switches of a kernel under tuning); part of the libraries' hash
 FLAGS += os.environ.get("QWEN3_RUNTIME_AMD_HIPCC_FLAGS", "").split()
 CORE_SOURCES = ["runtime.hip", "elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip", "attention_f32.hip", "sampling.hip",
-                "streams.hip", "moe.hip", "delta.hip", "combine.hip", "rotary.hip", "latent.hip", "retention.hip"]
+                "streams.hip", "moe.hip", "delta.hip", "combine.hip", "rotary.hip", "latent.hip", "retention.hip", "jointnorm.hip"]
 
 
 class BuildError(RuntimeError):

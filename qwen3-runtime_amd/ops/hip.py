@@ -101,6 +101,16 @@ class _RotateArgs(Structure):
         ("out", c_void_p), ("out_row", c_long), ("out_stride", c_int), ("out_offset", c_int),
         ("heads", c_int), ("width", c_int), ("pairs", c_int),
         ("positions", c_void_p), ("freq", c_void_p), ("scale_from_head", c_int), ("scale", c_float),
+        ("neighbours", c_int), ("magnitude", c_float),
+    ]
+
+
+class _JointNormArgs(Structure):
+    _fields_ = [
+        ("qk", c_void_p), ("row", c_long), ("bias", c_void_p), ("q_weight", c_void_p), ("k_weight", c_void_p),
+        ("positions", c_void_p), ("q_out", c_void_p), ("slots", c_void_p), ("k_cache", c_void_p), ("v_cache", c_void_p),
+        ("page_size", c_int), ("nq", c_int), ("nkv", c_int), ("d", c_int), ("values_are_keys", c_int),
+        ("eps", c_float), ("temp_coef", c_float), ("temp_every", c_int),
     ]
 
 
@@ -123,7 +133,7 @@ class _RuleArgs(Structure):
     ]
 
 
-ACTIVATIONS = {"swiglu": 0, "clamped": 1}
+ACTIVATIONS = {"swiglu": 0, "clamped": 1, "relu2": 2}  # relu2 has no gate
 
 
 def _planes(y, t, h, name):
@@ -325,6 +335,31 @@ class HipOps:
             c_float(eps), _ptr(rows), _ptr(out), _CODE[out_dtype], c_int(n_out), c_int(h), _stream()))
         return out
 
+    def scaled_add_rmsnorm(self, residual, parts, weight, eps, out_dtype, rows=None):
+        """``residual += sum_i scale_i * y_i`` in place, element by element (``parts``: up to four
+        (y, scale), ``y`` a matrix or float32 planes, ``scale`` float32 [H]), then the rows' RMS norm;
+        with ``rows`` only those, and ``residual`` is left alone."""
+        t, h = residual.shape
+        _need(residual, "residual", torch.float32)
+        _need(weight, "norm weight", torch.float32, (h,))
+        n = len(parts)
+        if not 1 <= n <= 4:
+            raise OpsError(f"a sum of {n} scaled outputs (1 to 4)")
+        ptrs, codes, counts, scales = (c_void_p * n)(), (c_int * n)(), (c_int * n)(), (c_void_p * n)()
+        for i, (y, scale) in enumerate(parts):
+            py, codes[i], counts[i] = _planes(y, t, h, "sub-layer output")
+            ptrs[i] = py.value if hasattr(py, "value") else py
+            scales[i] = _need(scale, "vector of a sub-layer's output", torch.float32, (h,)).data_ptr()
+        n_out = t
+        if rows is not None:
+            _need(rows, "rows", torch.int32)
+            n_out = rows.numel()
+        out = torch.empty((n_out, h), dtype=out_dtype, device=residual.device)
+        self._check(self.lib, self.lib.qrt_scaled_add_rmsnorm(
+            _ptr(residual), ptrs, codes, counts, scales, c_int(n), c_long(t * h), _ptr(weight), c_float(eps), _ptr(rows),
+            _ptr(out), _CODE[out_dtype], c_int(n_out), c_int(h), _stream()))
+        return out
+
     # ---- attention through a latent, retention ------------------------------------------
     def rmsnorm_columns(self, y, first, width, weight, eps):
         """The RMS norm of columns ``first .. first + width`` of ``y`` [T, W], [T, width] in ``y``'s type."""
@@ -338,9 +373,10 @@ class HipOps:
                                                            c_float(eps), _ptr(out), _CODE[y.dtype], c_int(t), _stream()))
         return out
 
-    def latent_store(self, y, first, rank, rot_dim, weight, eps, positions, freq, cache):
+    def latent_store(self, y, first, rank, rot_dim, weight, eps, positions, freq, cache, neighbours=False, magnitude=1.0):
         """Columns ``first .. first + rank`` of ``y`` RMS-normed (the latent ``c``) and the ``rot_dim``
-        columns behind them rotated (rotate-half over the first ``2 len(freq)``) go into the cache of
+        columns behind them rotated (rotate-half over the first ``2 len(freq)``; ``neighbours``: element
+        2i against 2i + 1; cosines and sines times ``magnitude``) go into the cache of
         one key/value head: the key row ``[c | k_rot]``, the value row ``[c | 0]``."""
         if cache is None:
             return
@@ -359,14 +395,15 @@ class HipOps:
         self._check(self.lib, self.lib.qrt_latent_store(
             _ptr(y), c_long(w), c_int(first), c_int(rank), c_int(rot_dim), _ptr(weight), c_float(eps), _ptr(positions),
             _ptr(freq), c_int(pairs), _ptr(cache.group.slots), _ptr(cache.k), _ptr(cache.v), c_int(cache.group.page_size),
-            c_long(pages), _CODE[y.dtype], c_int(t), _stream()))
+            c_long(pages), _CODE[y.dtype], c_int(t), c_int(bool(neighbours)), c_float(magnitude), _stream()))
 
     def rotate_half(self, x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq,
-                    scale_from_head=None, scale=1.0):
+                    scale_from_head=None, scale=1.0, neighbours=False, magnitude=1.0):
         """For every token and head copy ``width`` elements from ``x[t, h * in_stride + in_offset ...]`` to
         ``out[t, h * out_stride + out_offset ...]``, the first ``2 len(freq)`` of them turned (element i
         against element i + len(freq), by ``position * freq[i]``); heads from ``scale_from_head`` on are
-        multiplied by ``scale``. ``out`` may be float32 for a bfloat16 ``x``."""
+        multiplied by ``scale``. ``neighbours``: element 2i turns against element 2i + 1 instead; cosines and
+        sines are multiplied by ``magnitude``. ``out`` may be float32 for a bfloat16 ``x``."""
         t = x.shape[0]
         _need(x, "x")
         _need(out, "out", shape=(t, out.shape[1]))
@@ -379,6 +416,7 @@ class HipOps:
             a.freq = _need(freq, "freq", torch.float32, (pairs,)).data_ptr()
             a.positions = _need(positions, "positions", torch.int32, (t,)).data_ptr()
         a.scale_from_head, a.scale = heads if scale_from_head is None else scale_from_head, scale
+        a.neighbours, a.magnitude = int(bool(neighbours)), magnitude
         self._check(self.lib, self.lib.qrt_rotate_half(byref(a), _CODE[x.dtype], _CODE[out.dtype], c_int(t), _stream()))
         return out
 
@@ -423,6 +461,7 @@ class HipOps:
         a.x, a.x_row, a.in_stride, a.in_offset = y.data_ptr() + 2 * heads * dim * y.element_size(), w, vdim, 0
         a.out, a.out_row, a.out_stride, a.out_offset = out.data_ptr() + 2 * heads * dim * 4, c, vdim, 0
         a.heads, a.width, a.pairs, a.scale_from_head, a.scale = heads, vdim, 0, heads, 1.0
+        a.magnitude = 1.0
         self._check(self.lib, self.lib.qrt_rotate_half(byref(a), _CODE[y.dtype], F32, c_int(t), _stream()))
         return out
 
@@ -624,17 +663,22 @@ class HipOps:
         return out
 
     # ---- routed experts --------------------------------------------------------------
-    def route_top(self, x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None, group_score="top2"):
+    def route_top(self, x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None, group_score="top2",
+                  correction=None, renormalise=False, weight_scale=1.0):
         """Router logits ``x W^T + b`` in float32, the ``top`` largest per token and the softmax
         over those alone: (int32 [T, top], float32 [T, top]). ``scoring="sigmoid"``: the choice goes
         by ``sigmoid`` of the logits, which are also the weights, as they are; ``"softmax_all"``: by the
         softmax over all experts' logits, likewise. ``groups``, ``keep``: only experts of the ``keep``
         best of ``groups`` equal groups of neighbours can be chosen, a group's score being the sum of
-        its two largest entries (``group_score="top2"``) or its largest (``"max"``)."""
+        its two largest entries (``group_score="top2"``) or its largest (``"max"``). With scores over all
+        experts: ``correction`` [E] is added to them for the choice alone, ``renormalise`` divides the
+        chosen scores by their sum (+ 1e-20), ``weight_scale`` multiplies the weights at the end."""
         t, h = x.shape
         _need(x, "x")
         n = router.shape[0]
         _need(router, "router", torch.float32, (n, h))
+        if correction is not None:
+            _need(correction, "correction of the choice", torch.float32, (n,))
         if router_bias is not None:
             _need(router_bias, "router bias", torch.float32, (n,))
         index = torch.empty((t, top), dtype=torch.int32, device=x.device)
@@ -643,18 +687,20 @@ class HipOps:
                                                      _ptr(index), _ptr(weight), c_int(t), c_int(h), c_int(n),
                                                      c_int(top), c_int({"softmax_top": 0, "sigmoid": 1, "softmax_all": 2}[scoring]),
                                                      c_int(groups), c_int(groups if keep is None else keep),
-                                                     c_int(group_score == "max"), _stream()))
+                                                     c_int(group_score == "max"), _ptr(correction),
+                                                     c_int(bool(renormalise)), c_float(weight_scale), _stream()))
         return index, weight
 
     def moe_swiglu(self, x, gate_up, down, index, weight, activation="swiglu", limit=0.0, out=None):
         """``sum_j weight[t, j] * down[e] (silu(gate[e] x) * (up[e] x))`` with ``e = index[t, j]``;
-        ``gate_up`` [E, 2I, H] (gate rows first), ``down`` [E, H, I]. float32 [T, H]."""
+        ``gate_up`` [E, 2I, H] (gate rows first), ``down`` [E, H, I]. float32 [T, H]. ``activation="relu2"``:
+        experts without a gate, ``down[e] relu(up[e] x)^2``, and ``gate_up`` is the up rows alone, [E, I, H]."""
         t, h = x.shape
-        n, two_i, _ = gate_up.shape
-        inter = two_i // 2
+        n, rows_e, _ = gate_up.shape
+        inter = rows_e if activation == "relu2" else rows_e // 2
         top = index.shape[1]
         _need(x, "x")
-        _need(gate_up, "expert gate/up", x.dtype, (n, 2 * inter, h))
+        _need(gate_up, "expert gate/up", x.dtype, (n, rows_e, h))
         _need(down, "expert down", x.dtype, (n, h, inter))
         _need(index, "expert index", torch.int32, (t, top))
         _need(weight, "expert weight", torch.float32, (t, top))
@@ -728,14 +774,13 @@ class HipOps:
             # what bounds this form is the host's time per launch, so an expert costs two of them:
             # its products go straight into its rows of one buffer each (the library's for more
             # rows than the engine's own kernels take), and one activation kernel serves all experts
-            inter = gate_up.shape[1] // 2
-            both = torch.empty((pairs, 2 * inter), dtype=x.dtype, device=dev)
+            both = torch.empty((pairs, gate_up.shape[1]), dtype=x.dtype, device=dev)
             for e, a, b in busy:
                 if b - a > self.own_max_rows:
                     torch.mm(xs[a:b], gate_up[e].t(), out=both[a:b])
                 else:
                     both[a:b] = self.linear(xs[a:b], gate_up[e])
-            act = self.gated_act(both, activation, limit)
+            act = self.unary_act(both, activation) if activation == "relu2" else self.gated_act(both, activation, limit)
             for e, a, b in busy:
                 if b - a > self.own_max_rows:
                     torch.mm(act[a:b], down[e].t(), out=y[a:b])
@@ -743,7 +788,11 @@ class HipOps:
                     y[a:b] = self.linear(act[a:b], down[e])
         else:
             for e, a, b in busy:
-                y[a:b] = self.linear(self.gated_linear(xs[a:b], gate_up[e], activation, limit), down[e])
+                if activation == "relu2":
+                    act = self.unary_act(self.linear(xs[a:b], gate_up[e]), activation)
+                else:
+                    act = self.gated_linear(xs[a:b], gate_up[e], activation, limit)
+                y[a:b] = self.linear(act, down[e])
         self._check(self.lib, self.lib.qrt_moe_combine(_ptr(y), _ptr(place), _ptr(index), _ptr(offsets), c_int(padded),
                                                        _ptr(weight), _ptr(out), _CODE[x.dtype], c_int(t), c_int(h),
                                                        c_int(top), _stream()))
@@ -984,6 +1033,39 @@ class HipOps:
         else:
             a.nkv = a.nv = 0  # keys and values go nowhere: only queries are needed
         self._qk(a, qkv.dtype, pages)
+        return q
+
+    def qk_joint_norm_store(self, qk, nq, nkv, d, bias, q_w, k_w, eps, positions, q_temp, values_are_keys, cache):
+        """From the columns q | k (| v) of one product: biases (float32 over those columns, or None),
+        the RMS norm of all ``nq * d`` query elements of a token at once with weights of that size and
+        likewise of its ``nkv * d`` key elements, the queries times the temperature of their position
+        (``q_temp`` = (coef, every): ``1 + coef ln(floor((p + 1) / every) + 1)``; None: 1), and the write
+        of normed keys and raw values into the cache, the values being the biased keys themselves
+        (``values_are_keys``) or the v columns. Returns the queries [T, nq * d]."""
+        t, width = qk.shape
+        cols = (nq + (1 if values_are_keys else 2) * nkv) * d
+        _need(qk, "qk")
+        if width < cols:
+            raise OpsError(f"qk_joint_norm_store: rows of {width} for {cols} columns")
+        a = _JointNormArgs()
+        a.qk, a.row = qk.data_ptr(), width
+        if bias is not None:
+            if bias.numel() < cols:
+                raise OpsError(f"qk_joint_norm_store: {bias.numel()} biases for {cols} columns")
+            a.bias = _need(bias, "bias", torch.float32).data_ptr()
+        a.q_weight = _need(q_w, "q_norm", torch.float32, (nq * d,)).data_ptr()
+        a.k_weight = _need(k_w, "k_norm", torch.float32, (nkv * d,)).data_ptr()
+        a.positions = _need(positions, "positions", torch.int32, (t,)).data_ptr()
+        q = torch.empty((t, nq * d), dtype=qk.dtype, device=qk.device)
+        a.q_out, a.nq, a.nkv, a.d, a.values_are_keys, a.eps = q.data_ptr(), nq, nkv, d, int(bool(values_are_keys)), eps
+        if q_temp is not None:
+            a.temp_coef, a.temp_every = float(q_temp[0]), int(q_temp[1])
+        pages = 0
+        if cache is not None:
+            pages = self._check_cache(cache, nkv, d, qk.dtype)
+            a.slots = _need(cache.group.slots, "slots", torch.int32, (t,)).data_ptr()
+            a.k_cache, a.v_cache, a.page_size = cache.k.data_ptr(), cache.v.data_ptr(), cache.group.page_size
+        self._check(self.lib, self.lib.qrt_qk_joint_norm_store(byref(a), _CODE[qk.dtype], c_int(t), c_long(pages), _stream()))
         return q
 
     def qk_norm_split(self, qkv, nq, nkv, d, q_w, k_w, eps):

@@ -11,6 +11,7 @@ from .base import (  # noqa: F401
     NormedUpdate,
     Part,
     PositionEncoding,
+    ScaledUpdate,
     StepContext,
     StepCost,
     StreamUpdate,

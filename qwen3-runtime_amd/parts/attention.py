@@ -22,7 +22,13 @@ biases on the q, k and v projections (``bias``: tensors ``q_bias``, ``k_bias``, 
 product's output in float32, before any rotation); beside a window, the sequence's first
 ``keep_first`` tokens stay visible to every later query (key ``j`` is visible iff ``j <= i`` and
 ``i - j < window or j < keep_first``; the cache keeps their pages); a ``sink`` in the softmax, one more
-term of score 0 and no value in its denominator (``p_j = exp(s_j) / (1 + sum exp(s_j))``).
+term of score 0 and no value in its denominator (``p_j = exp(s_j) / (1 + sum exp(s_j))``); the q/k norm
+over the whole projection instead of per head (``qk_norm_scope="projection"``: all heads' query
+elements of a token are divided by their one root mean square, weights ``q_norm`` of that whole
+size, and likewise the keys); values that are the keys (``values_are_keys``: there is no ``v``
+projection, a key head's value is that head's key as projected, bias included, before any norm); a
+query temperature (``q_temp`` = (coef, every): the normed queries at position ``p`` are multiplied by
+``1 + coef * ln(floor((p + 1) / every) + 1)``, float32).
 """
 
 from __future__ import annotations
@@ -56,6 +62,9 @@ class GroupedQueryAttention(Mixer):
         bias: bool = False,
         keep_first: int = 0,
         sink: bool = False,
+        qk_norm_scope: str = "head",
+        values_are_keys: bool = False,
+        q_temp: tuple[float, int] | None = None,
         tensors=None,
     ):
         super().__init__(tensors)
@@ -80,6 +89,24 @@ class GroupedQueryAttention(Mixer):
         if self.keep_first < 0 or (self.keep_first and self.window is None):
             raise ValueError("first tokens are kept in sight beside a window")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        if qk_norm_scope not in ("head", "projection"):
+            raise ValueError(f"unknown scope of the q/k norm {qk_norm_scope!r} (head, projection)")
+        self.joint_norm = qk_norm_scope == "projection"
+        self.values_are_keys = bool(values_are_keys)
+        self.q_temp = None if q_temp is None else (float(q_temp[0]), int(q_temp[1]))
+        if self.q_temp is not None and self.q_temp[1] < 1:
+            raise ValueError(f"the query temperature counts positions in units of {self.q_temp[1]}")
+        if self.joint_norm:
+            # the form that one kernel serves: bias, norm over the projection, temperature, cache write
+            if (self.qk_norm_eps is None or not self.qk_norm_weight or position is not None or output_gate
+                    or self.value_dim != self.head_dim):
+                raise ValueError("the q/k norm over the whole projection has weights and an eps, and goes without "
+                                 "position encoding, output gate and values of another size than keys")
+        elif self.values_are_keys or self.q_temp is not None:
+            raise NotImplementedError("values that are the keys, and a query temperature, come with the q/k norm "
+                                      "over the whole projection")
+        if self.values_are_keys and self.value_dim != self.head_dim:
+            raise ValueError("values that are the keys have the keys' size")
         self.position = None
         if position is not None:
             self.position = part_class("position", position.kind)(**position.args, tensors=position.tensors)
@@ -98,29 +125,33 @@ class GroupedQueryAttention(Mixer):
         decls = [
             TensorDecl(self._name("q"), (self.num_heads * d, h)),
             TensorDecl(self._name("k"), (self.num_kv_heads * d, h)),
-            TensorDecl(self._name("v"), (self.num_kv_heads * dv, h)),
-            TensorDecl(self._name("o"), (h, self.num_heads * dv)),
         ]
+        if not self.values_are_keys:
+            decls.append(TensorDecl(self._name("v"), (self.num_kv_heads * dv, h)))
+        decls.append(TensorDecl(self._name("o"), (h, self.num_heads * dv)))
         if self.output_gate:
             decls.append(TensorDecl(self._name("g"), (self.num_heads * dv, h)))
         if self.has_bias:
             decls += [TensorDecl(self._name("q_bias"), (self.num_heads * d,)),
-                      TensorDecl(self._name("k_bias"), (self.num_kv_heads * d,)),
-                      TensorDecl(self._name("v_bias"), (self.num_kv_heads * dv,))]
+                      TensorDecl(self._name("k_bias"), (self.num_kv_heads * d,))]
+            if not self.values_are_keys:
+                decls.append(TensorDecl(self._name("v_bias"), (self.num_kv_heads * dv,)))
         if self.qk_norm_eps is not None and self.qk_norm_weight:
+            nq, nk = (self.num_heads, self.num_kv_heads) if self.joint_norm else (1, 1)
             decls += [
-                TensorDecl(self._name("q_norm"), (d,), init="norm"),
-                TensorDecl(self._name("k_norm"), (d,), init="norm"),
+                TensorDecl(self._name("q_norm"), (nq * d,), init="norm"),
+                TensorDecl(self._name("k_norm"), (nk * d,), init="norm"),
             ]
         return decls
 
     def load(self, fetch):
         # one product for q | k | v (| gate): the gate reads the same input
-        names = [self._name("q"), self._name("k"), self._name("v")] + ([self._name("g")] if self.output_gate else [])
+        names = [self._name("q"), self._name("k")] + ([] if self.values_are_keys else [self._name("v")]) \
+            + ([self._name("g")] if self.output_gate else [])
         self.qkv = fetch.fused(names, dim=0)
         self.o = fetch.matrix(self._name("o"))
         if self.has_bias:  # one vector over the product's columns; a gate's columns get zeros
-            pieces = [fetch.vector_f32(self._name(n)) for n in ("q_bias", "k_bias", "v_bias")]
+            pieces = [fetch.vector_f32(self._name(n)) for n in ("q_bias", "k_bias", "v_bias")[: 2 if self.values_are_keys else 3]]
             if self.output_gate:
                 pieces.append(torch.zeros(self.num_heads * self.value_dim, dtype=torch.float32, device=pieces[0].device))
             self.bias = fetch.constant(torch.cat(pieces))
@@ -131,7 +162,7 @@ class GroupedQueryAttention(Mixer):
             self.q_norm = self.k_norm = fetch.constant(torch.ones(self.head_dim, dtype=torch.float32))
 
     def step_cost(self, spans, rows, elem_bytes):
-        cost = super().step_cost(spans, rows, elem_bytes)  # the four projections
+        cost = super().step_cost(spans, rows, elem_bytes)  # the projections
         for q, kv in spans:  # scores and weighted values: 4 D operations per (query head, visible key)
             first = kv - q
             if self.window:
@@ -148,6 +179,15 @@ class GroupedQueryAttention(Mixer):
         nq, nkv, d, dv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
         qkv = ops.linear(x, self.qkv)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
+        if self.joint_norm:
+            # biases, the norm over each whole projection, the queries' temperature and the cache
+            # write (keys normed, values raw: the keys themselves, or the v columns) in one pass
+            q = ops.qk_joint_norm_store(qkv, nq, nkv, d, self.bias, self.q_norm, self.k_norm, eps, ctx.positions,
+                                        self.q_temp, self.values_are_keys, cache if cache.writes else None)
+            more = {name: value for name, value in (("chunk", self.chunk), ("softcap", self.softcap),
+                                                    ("keep_first", self.keep_first), ("sink", self.sink)) if value}
+            attn = ops.paged_attention(q, cache, ctx, nq, nkv, d, self.scale, self.window, **more)
+            return ops.linear_for_residual(attn, self.o)
         in_place = getattr(self.position, "in_place", False)
         if in_place:
             # biases and an encoding that works on the product where it lies: after it the mixer

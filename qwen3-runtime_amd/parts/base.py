@@ -186,6 +186,15 @@ class NormedUpdate:
 
 
 @dataclass
+class ScaledUpdate:
+    """Several sub-layer outputs that join the residual stream in one sum, each times a vector of
+    its own, element by element: ``x <- x + sum_i scale_i * y_i``. Like a plain ``delta`` it is
+    applied by the norm that comes next."""
+
+    parts: list  # of (y, scale): y [T, H] or float32 planes [P, T, H] whose sum it is; scale float32 [H]
+
+
+@dataclass
 class GroupView:
     """One cache group's view of this step's batch (device tensors).
 

@@ -1,5 +1,6 @@
 """Arrangements of a layer's parts: the pre-norm residual block, over one residual stream or
-over several (hyper-connections), and the block with a norm on both sides of each sub-layer.
+over several (hyper-connections), the block with a norm on both sides of each sub-layer, and
+the block whose mixer and feed-forward read one norm and join the stream in one scaled sum.
 
 ``x += mixer(norm_in(x)); x += feed_forward(norm_post(x))``: the form the
 reference's oracle writes (tests/cpu/reference_qwen3.py:79-110) and its model
@@ -12,7 +13,7 @@ with the norm that follows it without a block knowing its neighbour.
 from __future__ import annotations
 
 from ..registry import register_part
-from .base import Block, NormedUpdate, StreamUpdate
+from .base import Block, NormedUpdate, ScaledUpdate, StreamUpdate
 from .plan import TensorDecl
 
 
@@ -131,3 +132,53 @@ class HyperConnectionBlock(Block):
             return residual, pending
         x = self.norm_post.forward(ctx, residual, pending, read=c["in2"])
         return residual, StreamUpdate(self.feed_forward.forward(ctx, x), c["mix2"], c["out2"])
+
+
+@register_part("block", "parallel_scaled")
+class ParallelScaledBlock(Block):
+    """Mixer and feed-forward side by side: one norm, ``n = norm_in(x)``, both read it, and
+    ``x <- x + s1 * mixer(n) + s2 * feed_forward(n)`` with a vector per sub-layer (tensors ``scale1``,
+    ``scale2``; ``layer_scale=False``: no vectors, the plain sum). The two outputs go on as one
+    ``ScaledUpdate``, which the next layer's norm adds in the pass in which it normalises. A block
+    without feed-forward has the first term only."""
+
+    norm_names = ("input",)
+
+    def __init__(self, mixer, feed_forward, norms, hidden_size: int, layer_scale: bool = True, tensors=None):
+        super().__init__(tensors)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norm_in = norms["input"]
+        self.hidden_size, self.layer_scale = int(hidden_size), bool(layer_scale)
+        self.scale1 = self.scale2 = None
+
+    def children(self):
+        return tuple(p for p in (self.norm_in, self.mixer, self.feed_forward) if p is not None)
+
+    def tensor_decls(self):
+        if not self.layer_scale:
+            return []
+        names = ("scale1",) if self.feed_forward is None else ("scale1", "scale2")
+        return [TensorDecl(self._name(n), (self.hidden_size,), init="norm") for n in names]
+
+    def load(self, fetch):
+        if self.layer_scale:
+            self.scale1 = fetch.vector_f32(self._name("scale1"))
+            if self.feed_forward is not None:
+                self.scale2 = fetch.vector_f32(self._name("scale2"))
+        else:
+            import torch
+
+            self.scale1 = self.scale2 = fetch.constant(torch.ones(self.hidden_size, dtype=torch.float32))
+
+    def step_cost(self, spans, rows, elem_bytes):
+        cost = super().step_cost(spans, rows, elem_bytes)
+        cost.flop = 0.0  # vectors, not matrices that multiply tokens
+        return cost
+
+    def forward(self, ctx, residual, delta, cache):
+        x = self.norm_in.forward(ctx, residual, delta)
+        parts = [(self.mixer.forward(ctx, x, cache), self.scale1)]
+        if self.feed_forward is not None:
+            parts.append((self.feed_forward.forward(ctx, x), self.scale2))
+        return residual, ScaledUpdate(parts)

@@ -16,7 +16,11 @@ experts of the ``keep`` best groups can be chosen. ``activation="clamped"`` with
 ``limit``: ``g = min(gate x, limit)``, ``u = clamp(up x, -limit, limit)``, ``y = g sigmoid(1.702 g) (u + 1)``
 in place of ``silu(g) u``. ``shared_size``: one more expert of that inner width (tensors
 ``shared_gate``, ``shared_up``, ``shared_down``; ``shared_limit`` its clamp) that every token passes
-and whose output is added unweighted.
+and whose output is added unweighted. ``correction`` (with ``softmax_all`` or ``sigmoid`` scores): a
+tensor ``correction`` [experts] is added to the scores for the choice alone; the weights are the
+chosen experts' scores without it. ``renormalise``: the chosen scores are divided by their sum
+(plus 1e-20). ``weight_scale``: the weights are multiplied by it at the end.
+``activation="relu2"``: experts without a gate, ``down_e( relu(up_e(x))^2 )``, tensors ``up`` and ``down``.
 """
 
 from __future__ import annotations
@@ -35,7 +39,8 @@ class RoutedSwiGLU(FeedForward):
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
                  router_bias: bool = True, scoring: str = "softmax_top", groups: int = 1, keep: int | None = None,
                  activation: str = "swiglu", limit: float = 0.0, shared_size: int | None = None,
-                 shared_limit: float | None = None, group_score: str = "top2", tensors=None):
+                 shared_limit: float | None = None, group_score: str = "top2", correction: bool = False,
+                 renormalise: bool = False, weight_scale: float = 1.0, tensors=None):
         super().__init__(tensors)
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
@@ -44,12 +49,18 @@ class RoutedSwiGLU(FeedForward):
         if not 1 <= self.top <= self.num_experts:
             raise ValueError(f"each token takes {self.top} of {self.num_experts} experts")
         self.has_router_bias = bool(router_bias)
-        if scoring not in ("softmax_top", "sigmoid", "softmax_all") or activation not in ("swiglu", "clamped") \
+        if scoring not in ("softmax_top", "sigmoid", "softmax_all") or activation not in ("swiglu", "clamped", "relu2") \
                 or group_score not in ("top2", "max"):
             raise ValueError(f"unknown scoring {scoring!r} (softmax_top, sigmoid, softmax_all), activation {activation!r} "
-                             f"(swiglu, clamped) or group score {group_score!r} (top2, max)")
+                             f"(swiglu, clamped, relu2) or group score {group_score!r} (top2, max)")
         self.scoring, self.activation, self.limit = scoring, activation, float(limit)
         self.group_score = group_score
+        self.gated = activation != "relu2"
+        self.has_correction, self.renormalise, self.weight_scale = bool(correction), bool(renormalise), float(weight_scale)
+        if (self.has_correction or self.renormalise) and scoring == "softmax_top":
+            raise ValueError("a correction of the choice and renormalised weights go with scores over all experts")
+        if not self.gated and shared_size:
+            raise NotImplementedError("a shared expert beside experts without a gate")
         self.groups = int(groups)
         self.keep = self.groups if keep is None else int(keep)
         if self.groups < 1 or self.num_experts % self.groups or not 1 <= self.keep <= self.groups:
@@ -59,7 +70,7 @@ class RoutedSwiGLU(FeedForward):
         self.shared_size = None if shared_size is None else int(shared_size)
         self.shared_limit = self.limit if shared_limit is None else float(shared_limit)
         self.router = self.router_bias = self.gate_up = self.down = None
-        self.shared_gate_up = self.shared_down = None
+        self.shared_gate_up = self.shared_down = self.correction = None
 
     def _expert(self, logical: str, e: int) -> str:
         return self._name(logical).format(e=e)
@@ -70,8 +81,10 @@ class RoutedSwiGLU(FeedForward):
         if self.has_router_bias:
             decls.append(TensorDecl(self._name("router_bias"), (self.num_experts,)))
         for e in range(self.num_experts):
-            decls += [TensorDecl(self._expert("gate", e), (i, h)), TensorDecl(self._expert("up", e), (i, h)),
-                      TensorDecl(self._expert("down", e), (h, i))]
+            decls += ([TensorDecl(self._expert("gate", e), (i, h))] if self.gated else []) + \
+                     [TensorDecl(self._expert("up", e), (i, h)), TensorDecl(self._expert("down", e), (h, i))]
+        if self.has_correction:
+            decls.append(TensorDecl(self._name("correction"), (self.num_experts,)))
         if self.shared_size:
             s = self.shared_size
             decls += [TensorDecl(self._name("shared_gate"), (s, h)), TensorDecl(self._name("shared_up"), (s, h)),
@@ -84,8 +97,11 @@ class RoutedSwiGLU(FeedForward):
         self.router = fetch.vector_f32(self._name("router"))
         if self.has_router_bias:
             self.router_bias = fetch.vector_f32(self._name("router_bias"))
-        names = [self._expert(part, e) for e in range(n) for part in ("gate", "up")]
-        self.gate_up = fetch.fused(names, dim=0).view(n, 2 * i, h)
+        if self.has_correction:
+            self.correction = fetch.vector_f32(self._name("correction"))
+        halves = ("gate", "up") if self.gated else ("up",)  # without a gate the tensor holds the up rows alone
+        names = [self._expert(part, e) for e in range(n) for part in halves]
+        self.gate_up = fetch.fused(names, dim=0).view(n, len(halves) * i, h)
         self.down = fetch.fused([self._expert("down", e) for e in range(n)], dim=0).view(n, h, i)
         if self.shared_size:
             self.shared_gate_up = fetch.fused([self._name("shared_gate"), self._name("shared_up")], dim=0)
@@ -99,9 +115,9 @@ class RoutedSwiGLU(FeedForward):
         cost = StepCost()
         cost.weight_bytes[self._name("router")] = n * h * 4
         for e in range(used):  # which ones is not known here: the first `used` stand for them
-            for part, size in (("gate", i * h), ("up", i * h), ("down", h * i)):
+            for part, size in (("gate", i * h), ("up", i * h), ("down", h * i))[0 if self.gated else 1:]:
                 cost.weight_bytes[self._expert(part, e)] = size * elem_bytes
-        cost.flop = 2.0 * tokens * (n * h + self.top * 3 * h * i)
+        cost.flop = 2.0 * tokens * (n * h + self.top * (3 if self.gated else 2) * h * i)
         if self.shared_size:
             for part in ("shared_gate", "shared_up", "shared_down"):
                 cost.weight_bytes[self._name(part)] = self.shared_size * h * elem_bytes
@@ -115,6 +131,8 @@ class RoutedSwiGLU(FeedForward):
             index, weight = ops.route_top(x, self.router, self.router_bias, self.top)
             return ops.moe_swiglu(x, self.gate_up, self.down, index, weight)
         how = {"group_score": self.group_score} if self.group_score != "top2" else {}
+        if self.has_correction or self.renormalise or self.weight_scale != 1.0:
+            how.update(correction=self.correction, renormalise=self.renormalise, weight_scale=self.weight_scale)
         index, weight = ops.route_top(x, self.router, self.router_bias, self.top, scoring=self.scoring,
                                       groups=self.groups, keep=self.keep, **how)
         more = {"activation": self.activation, "limit": self.limit}

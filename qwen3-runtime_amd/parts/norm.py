@@ -13,7 +13,8 @@ squared deviations, float32.
 Either norm also serves several residual streams ``[T, S, H]`` (hyper-connections): the update
 that is pending is then a ``StreamUpdate`` (the streams mixed among themselves plus the
 sub-layer's output times a weight per stream), and what is normalised is the sum of the
-streams weighted by ``read``; a norm built with ``streams=S`` and called without ``read`` takes
+streams weighted by ``read``; a ``ScaledUpdate`` (the outputs of sub-layers that ran side by side,
+each times a vector) joins one stream as ``x + sum_i s_i * y_i``; a norm built with ``streams=S`` and called without ``read`` takes
 the plain sum (the model's last norm).
 """
 
@@ -22,7 +23,7 @@ from __future__ import annotations
 import torch
 
 from ..registry import register_part
-from .base import Norm, NormedUpdate
+from .base import Norm, NormedUpdate, ScaledUpdate
 from .plan import TensorDecl
 
 
@@ -69,6 +70,11 @@ class RMSNorm(Norm):
                 raise NotImplementedError("a normed update meets the plain RMS norm only")
             return ctx.ops.add_rmsnorm(residual, delta.y, self.weight, self.eps, ctx.dtype, rows,
                                        delta_norm=(delta.weight, delta.eps))
+        if isinstance(delta, ScaledUpdate):
+            # outputs of sub-layers that ran side by side, each times its vector
+            if self.has_bias or self.delta_scale != 1.0:
+                raise NotImplementedError("a sum of scaled updates meets the plain RMS norm only")
+            return ctx.ops.scaled_add_rmsnorm(residual, delta.parts, self.weight, self.eps, ctx.dtype, rows)
         if self.has_bias:
             return ctx.ops.mix_norm(residual, delta, None, self.weight, self.bias, self.eps, ctx.dtype, rows)
         if self.delta_scale != 1.0:

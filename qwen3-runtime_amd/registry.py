@@ -137,3 +137,4 @@ def _load_builtin() -> None:
     from .models import deginex  # noqa: F401  (registers Deginex)
     from .models import zisedra  # noqa: F401  (registers Zisedra)
     from .models import roserax  # noqa: F401  (registers Roserax)
+    from .models import zuvasun  # noqa: F401  (registers Zuvasun)

@@ -212,17 +212,22 @@ def mix_norm(streams, update, read, weight, bias, eps, out_dtype, rows=None, com
     return y.to(out_dtype)
 
 
-def route_top(x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None, group_score="top2"):
+def route_top(x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None, group_score="top2",
+              correction=None, renormalise=False, weight_scale=1.0):
     """float32 logits x W^T + b; the ``top`` largest per token (ties: the lower index first) and
     the softmax over those alone. Returns (int32 [T, top], float32 [T, top]). With sigmoid scoring
-    the scores are the weights; with groups only the best ``keep`` groups' experts can be chosen."""
+    the scores are the weights; with groups only the best ``keep`` groups' experts can be chosen.
+    ``correction`` [E] is added to the scores for the choice alone; ``renormalise`` divides the chosen
+    scores by their sum (+ 1e-20); ``weight_scale`` multiplies the weights at the end."""
     logits = x.to(torch.float32) @ router.to(torch.float32).T
     if router_bias is not None:
         logits = logits + router_bias.to(torch.float32)
     values = torch.sigmoid(logits) if scoring == "sigmoid" else \
         torch.softmax(logits, dim=-1) if scoring == "softmax_all" else logits
-    pick = values
+    pick = values if correction is None else values + correction.to(torch.float32)
     if groups > 1 and keep is not None and keep < groups:
+        if correction is not None:
+            raise NotImplementedError("groups of experts beside a correction of the choice")
         t, e = values.shape
         per = e // groups
         g = values.view(t, groups, per)
@@ -232,7 +237,12 @@ def route_top(x, router, router_bias, top, scoring="softmax_top", groups=1, keep
         pick = torch.where(stay[:, :, None].expand(t, groups, per).reshape(t, e), values,
                            torch.full_like(values, float("-inf")))
     best, index = torch.topk(pick, top, dim=-1)
-    return index.to(torch.int32), best if scoring != "softmax_top" else torch.softmax(best, dim=-1)
+    if scoring == "softmax_top":
+        return index.to(torch.int32), torch.softmax(best, dim=-1)
+    weight = torch.gather(values, 1, index)
+    if renormalise:
+        weight = weight / (weight.sum(-1, keepdim=True) + 1e-20)
+    return index.to(torch.int32), weight * weight_scale if weight_scale != 1.0 else weight
 
 
 def gated(g, u, activation="swiglu", limit=0.0):
@@ -253,7 +263,10 @@ def moe_swiglu(x, gate_up, down, index, weight, compute=torch.float32, activatio
         for e in index[:, j].unique().tolist():
             sel = (index[:, j] == e).nonzero()[:, 0]
             gu = (xc[sel] @ gate_up[e].to(compute).T).to(x.dtype).to(compute)
-            act = gated(gu[:, :inter], gu[:, inter:], activation, limit).to(x.dtype).to(compute)
+            if activation == "relu2":  # no gate: the tensor holds the up rows alone
+                act = torch.relu(gu).pow(2).to(x.dtype).to(compute)
+            else:
+                act = gated(gu[:, :inter], gu[:, inter:], activation, limit).to(x.dtype).to(compute)
             out[sel] += weight[sel, j, None] * (act @ down[e].to(compute).T).to(torch.float32)
     return out
 
@@ -356,18 +369,25 @@ def argmax(logits):
     return torch.argmax(logits, dim=-1).to(torch.int32)
 
 
-def rotate_half_copy(x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq):
+def rotate_half_copy(x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq,
+                     neighbours=False, magnitude=1.0):
     """For every token and head copy ``width`` elements from ``x[t, h * in_stride + in_offset ...]`` to
     ``out[t, h * out_stride + out_offset ...]``, the first ``2 len(freq)`` of them turned: element i
-    against element i + len(freq), by ``position * freq[i]`` (float32 angles)."""
+    against element i + len(freq) (``neighbours``: element 2i against element 2i + 1), by
+    ``position * freq[i]`` (float32 angles), cosines and sines times ``magnitude``."""
     t = x.shape[0]
     src = x[:, : heads * in_stride].reshape(t, heads, in_stride)[:, :, in_offset: in_offset + width].to(torch.float32)
     n = 0 if freq is None else freq.numel()
     if n:
         ang = positions.to(torch.float32)[:, None] * freq.to(torch.float32)[None, :]
-        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
-        u, v = src[..., :n], src[..., n: 2 * n]
-        src = torch.cat([u * cos - v * sin, v * cos + u * sin, src[..., 2 * n:]], dim=-1)
+        cos, sin = ang.cos()[:, None, :] * magnitude, ang.sin()[:, None, :] * magnitude
+        if neighbours:
+            u, v = src[..., 0: 2 * n: 2], src[..., 1: 2 * n: 2]
+            turned = torch.stack([u * cos - v * sin, v * cos + u * sin], dim=-1).flatten(-2)
+            src = torch.cat([turned, src[..., 2 * n:]], dim=-1)
+        else:
+            u, v = src[..., :n], src[..., n: 2 * n]
+            src = torch.cat([u * cos - v * sin, v * cos + u * sin, src[..., 2 * n:]], dim=-1)
     out[:, : heads * out_stride].view(t, heads, out_stride)[:, :, out_offset: out_offset + width] = src.to(out.dtype)
     return out
 
@@ -377,14 +397,15 @@ def rmsnorm_columns(y, first, width, weight, eps):
     return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight).to(y.dtype)
 
 
-def latent_store(y, first, rank, rot_dim, weight, eps, positions, freq, k_cache, v_cache, slots, page_size):
+def latent_store(y, first, rank, rot_dim, weight, eps, positions, freq, k_cache, v_cache, slots, page_size,
+                 neighbours=False, magnitude=1.0):
     """Columns ``first .. first + rank`` of ``y`` RMS-normed (the latent) and the ``rot_dim`` behind them
     rotated: the key row ``[c | k_rot]`` and the value row ``[c | 0]`` of one key/value head."""
     t = y.shape[0]
     c = rmsnorm_columns(y, first, rank, weight, eps).to(torch.float32)
     rot = torch.empty((t, rot_dim), dtype=torch.float32, device=y.device)
     rotate_half_copy(y[:, first + rank: first + rank + rot_dim].contiguous(), rot_dim, 0, rot, rot_dim, 0, 1, rot_dim,
-                     positions, freq)
+                     positions, freq, neighbours, magnitude)
     k = torch.cat([c, rot], dim=1)[:, None, :]
     v = torch.cat([c, torch.zeros_like(rot)], dim=1)[:, None, :]
     kv_store(k, v, k_cache, v_cache, slots, page_size)
@@ -394,9 +415,9 @@ def heads_linear(x, in_stride, in_offset, w, out, out_stride, out_offset, comput
     """Per head h: out[t, h * out_stride + out_offset + n] = sum_k w[h, n, k] x[t, h * in_stride + in_offset + k]."""
     t = x.shape[0]
     heads, n, k = w.shape
-    src = x.view(t, heads, in_stride)[:, :, in_offset: in_offset + k].to(compute)
+    src = x[:, : heads * in_stride].reshape(t, heads, in_stride)[:, :, in_offset: in_offset + k].to(compute)
     res = torch.einsum("thk,hnk->thn", src, w.to(compute))
-    out.view(t, heads, out_stride)[:, :, out_offset: out_offset + n] = res.to(out.dtype)
+    out[:, : heads * out_stride].view(t, heads, out_stride)[:, :, out_offset: out_offset + n] = res.to(out.dtype)
     return out
 
 
@@ -434,6 +455,40 @@ def unary_act(x, kind):
     return torch.relu(x.to(torch.float32)).pow(2).to(x.dtype)
 
 
+def scaled_add_rmsnorm(residual, parts, weight, eps, out_dtype, rows=None, compute=torch.float32):
+    """``residual += sum_i scale_i * y_i`` in place (each ``y_i`` a matrix or planes), then the rows' RMS
+    norm; with ``rows`` only those, and ``residual`` is left alone."""
+    total = None
+    for y, scale in parts:
+        term = planes_sum(y) * scale.to(torch.float32)
+        total = term if total is None else total + term
+    return add_rmsnorm(residual, total, weight, eps, out_dtype, rows, compute)
+
+
+def qk_joint_norm_store(qk, nq, nkv, d, bias, q_w, k_w, eps, positions, q_temp, values_are_keys,
+                        k_cache=None, v_cache=None, slots=None, page_size=None):
+    """Columns q | k (| v) of a product: biases added in float32; the values are the keys as they
+    then are (or the v columns); all query elements of a token are divided by their one root
+    mean square and multiplied by ``q_w`` [nq d], likewise the keys with ``k_w`` [nkv d]; queries at
+    position p times ``1 + coef ln(floor((p + 1) / every) + 1)``; keys and values go to the cache."""
+    t = qk.shape[0]
+    y = qk.to(torch.float32)
+    if bias is not None:
+        y = y + bias
+    q, k = y[:, : nq * d], y[:, nq * d: (nq + nkv) * d]
+    v = k if values_are_keys else y[:, (nq + nkv) * d: (nq + 2 * nkv) * d]
+    v = v.to(qk.dtype)
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_w
+    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_w
+    if q_temp is not None:
+        coef, every = q_temp
+        p = positions.to(torch.float32)
+        q = q * (1.0 + coef * torch.log(torch.floor((p + 1.0) / every) + 1.0))[:, None]
+    if k_cache is not None:
+        kv_store(k.view(t, nkv, d), v.view(t, nkv, d), k_cache, v_cache, slots, page_size)
+    return q.to(qk.dtype)
+
+
 class TorchOps:
     """The engine's op interface over the functions above (tests only)."""
 
@@ -455,16 +510,27 @@ class TorchOps:
     def rmsnorm_columns(self, y, first, width, weight, eps):
         return rmsnorm_columns(y, first, width, weight, eps)
 
-    def latent_store(self, y, first, rank, rot_dim, weight, eps, positions, freq, cache):
+    def latent_store(self, y, first, rank, rot_dim, weight, eps, positions, freq, cache, neighbours=False, magnitude=1.0):
         if cache is not None:
             latent_store(y, first, rank, rot_dim, weight, eps, positions, freq, cache.k, cache.v, cache.group.slots,
-                         cache.group.page_size)
+                         cache.group.page_size, neighbours, magnitude)
+
+    def scaled_add_rmsnorm(self, residual, parts, weight, eps, out_dtype, rows=None):
+        return scaled_add_rmsnorm(residual, parts, weight, eps, out_dtype, rows, self.compute)
+
+    def qk_joint_norm_store(self, qk, nq, nkv, d, bias, q_w, k_w, eps, positions, q_temp, values_are_keys, cache):
+        if cache is None:
+            return qk_joint_norm_store(qk, nq, nkv, d, bias, q_w, k_w, eps, positions, q_temp, values_are_keys)
+        return qk_joint_norm_store(qk, nq, nkv, d, bias, q_w, k_w, eps, positions, q_temp, values_are_keys,
+                                   cache.k, cache.v, cache.group.slots, cache.group.page_size)
 
     def heads_linear(self, x, in_stride, in_offset, w, out, out_stride, out_offset):
         return heads_linear(x, in_stride, in_offset, w, out, out_stride, out_offset, self.compute)
 
-    def rotate_half(self, x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq):
-        return rotate_half_copy(x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq)
+    def rotate_half(self, x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq,
+                    neighbours=False, magnitude=1.0):
+        return rotate_half_copy(x, in_stride, in_offset, out, out_stride, out_offset, heads, width, positions, freq,
+                                neighbours, magnitude)
 
     def sigmoid_gate(self, out, gate):
         out.copy_((out.to(torch.float32) * torch.sigmoid(gate.to(torch.float32))).to(out.dtype))
@@ -528,8 +594,10 @@ class TorchOps:
     def mix_norm(self, streams, update, read, weight, bias, eps, out_dtype, rows=None):
         return mix_norm(streams, update, read, weight, bias, eps, out_dtype, rows, self.compute)
 
-    def route_top(self, x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None, group_score="top2"):
-        return route_top(x, router, router_bias, top, scoring, groups, keep, group_score)
+    def route_top(self, x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None, group_score="top2",
+                  correction=None, renormalise=False, weight_scale=1.0):
+        return route_top(x, router, router_bias, top, scoring, groups, keep, group_score, correction, renormalise,
+                         weight_scale)
 
     def moe_swiglu(self, x, gate_up, down, index, weight, activation="swiglu", limit=0.0):
         return moe_swiglu(x, gate_up, down, index, weight, self.compute, activation, limit)
