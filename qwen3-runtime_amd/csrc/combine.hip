@@ -249,21 +249,20 @@ struct ScaledTerms {
   int count;
 };
 
+template <int N>
 __device__ __forceinline__ float scaled_sum_at(const ScaledTerms& s, float x, size_t at, int i) {
-  float part[SA_TERMS], sc[SA_TERMS];
+  float part[N], sc[N];
 #pragma unroll
-  for (int k = 0; k < SA_TERMS; ++k) {
-    const int kk = k < s.count ? k : 0;
-    part[k] = planes_at(s.y[kk], at);
-    sc[k] = s.scale[kk][i];
+  for (int k = 0; k < N; ++k) {
+    part[k] = planes_at(s.y[k], at);
+    sc[k] = s.scale[k][i];
   }
 #pragma unroll
-  for (int k = 0; k < SA_TERMS; ++k)
-    if (k < s.count) x = fmaf(sc[k], part[k], x);
+  for (int k = 0; k < N; ++k) x = fmaf(sc[k], part[k], x);
   return x;
 }
 
-template <typename TO>
+template <typename TO, int N>
 __global__ __launch_bounds__(1024) void scaled_add_rmsnorm_kernel(float* __restrict__ residual, ScaledTerms s,
                                                                   const float* __restrict__ weight, float eps,
                                                                   const int* __restrict__ rows, TO* __restrict__ out,
@@ -276,7 +275,7 @@ __global__ __launch_bounds__(1024) void scaled_add_rmsnorm_kernel(float* __restr
 #pragma unroll
   for (int j = 0; j < NM_KEEP; ++j) {
     const int i = min((int)threadIdx.x + 1024 * j, hidden - 1);
-    vx[j] = scaled_sum_at(s, residual[row + i], row + i, i);
+    vx[j] = scaled_sum_at<N>(s, residual[row + i], row + i, i);
     wn[j] = weight[i];
   }
   float sx = 0.f;
@@ -289,7 +288,7 @@ __global__ __launch_bounds__(1024) void scaled_add_rmsnorm_kernel(float* __restr
     }
   }
   for (int i = threadIdx.x + 1024 * NM_KEEP; i < hidden; i += 1024) {
-    const float x = scaled_sum_at(s, residual[row + i], row + i, i);
+    const float x = scaled_sum_at<N>(s, residual[row + i], row + i, i);
     sx += x * x;
     if (!rows) residual[row + i] = x;
   }
@@ -301,7 +300,7 @@ __global__ __launch_bounds__(1024) void scaled_add_rmsnorm_kernel(float* __restr
     if (i < hidden) out[(size_t)b * hidden + i] = from_f32<TO>(vx[j] * ix * wn[j]);
   }
   for (int i = threadIdx.x + 1024 * NM_KEEP; i < hidden; i += 1024) {
-    const float x = rows ? scaled_sum_at(s, residual[row + i], row + i, i) : residual[row + i];
+    const float x = rows ? scaled_sum_at<N>(s, residual[row + i], row + i, i) : residual[row + i];
     out[(size_t)b * hidden + i] = from_f32<TO>(x * ix * weight[i]);
   }
 }
@@ -322,11 +321,17 @@ extern "C" int qrt_scaled_add_rmsnorm(float* residual, const void* const* y, con
     s.scale[k] = scale[kk];
   }
   if (num_out == 0) return 0;
-  if (out_dtype == QRT_F32)
-    scaled_add_rmsnorm_kernel<float><<<num_out, 1024, 0, stream>>>(residual, s, weight, eps, rows, (float*)out, hidden);
-  else if (out_dtype == QRT_BF16)
-    scaled_add_rmsnorm_kernel<bf16_t><<<num_out, 1024, 0, stream>>>(residual, s, weight, eps, rows, (bf16_t*)out, hidden);
-  else return qrt_fail("scaled_add_rmsnorm: unknown dtype %d", out_dtype);
+  QRT_CHECK(out_dtype == QRT_F32 || out_dtype == QRT_BF16, "scaled_add_rmsnorm: unknown dtype %d", out_dtype);
+#define SA_LAUNCH(N)                                                                                                          \
+  if (out_dtype == QRT_F32)                                                                                                   \
+    scaled_add_rmsnorm_kernel<float, N><<<num_out, 1024, 0, stream>>>(residual, s, weight, eps, rows, (float*)out, hidden);   \
+  else                                                                                                                        \
+    scaled_add_rmsnorm_kernel<bf16_t, N><<<num_out, 1024, 0, stream>>>(residual, s, weight, eps, rows, (bf16_t*)out, hidden)
+  if (count == 1) { SA_LAUNCH(1); }
+  else if (count == 2) { SA_LAUNCH(2); }
+  else if (count == 3) { SA_LAUNCH(3); }
+  else { SA_LAUNCH(4); }
+#undef SA_LAUNCH
   QRT_LAUNCH_CHECK("scaled_add_rmsnorm");
   return 0;
 }

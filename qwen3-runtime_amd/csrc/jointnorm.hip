@@ -24,33 +24,46 @@ struct JointNormArgs {
   float eps, temp_coef; int temp_every;  // temp_every 0: no temperature
 };
 
-template <typename T>
-__global__ __launch_bounds__(256) void joint_norm_kernel(JointNormArgs a) {
+// Two sums over a block of up to 1,024 threads at once; every thread gets both, added in the same order.
+__device__ __forceinline__ void block_sum_pair(float& x, float& y, float* red) {
+  x = wave_sum(x);
+  y = wave_sum(y);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = (blockDim.x + 63) >> 6;
+  if (lane == 0) { red[wave] = x; red[16 + wave] = y; }
+  __syncthreads();
+  x = y = 0.f;
+  for (int i = 0; i < nw; ++i) { x += red[i]; y += red[16 + i]; }
+}
+
+// THREADS a block: 1,024 for steps of few tokens (a token's row is then through in one or two
+// rounds of loads), 256 for many.
+template <typename T, int THREADS>
+__global__ __launch_bounds__(THREADS) void joint_norm_kernel(JointNormArgs a) {
   extern __shared__ float sm[];  // [(nq + nkv) * d], then 32 for the sums
   const int t = blockIdx.x;
   const int wq = a.nq * a.d, wk = a.nkv * a.d;
   float* red = sm + wq + wk;
   const T* row = (const T*)a.qk + (size_t)t * a.row;
   float sq = 0.f, sk = 0.f;
-  for (int i = threadIdx.x; i < wq + wk; i += 256) {
+  for (int i = threadIdx.x; i < wq + wk; i += THREADS) {
     const float v = to_f32<T>(row[i]) + (a.bias ? a.bias[i] : 0.f);
     sm[i] = v;
     if (i < wq) sq += v * v; else sk += v * v;
   }
-  sq = block_sum(sq, red);
-  sk = block_sum(sk, red);
+  block_sum_pair(sq, sk, red);
   const float iq = 1.0f / sqrtf(sq / (float)wq + a.eps);
   const float ik = 1.0f / sqrtf(sk / (float)wk + a.eps);
   float temp = 1.0f;
   if (a.temp_every > 0) temp = 1.0f + a.temp_coef * logf((float)((a.positions[t] + 1) / a.temp_every + 1));
   T* qo = (T*)a.q_out + (size_t)t * wq;
-  for (int i = threadIdx.x; i < wq; i += 256) qo[i] = from_f32<T>(sm[i] * iq * a.q_weight[i] * temp);
+  for (int i = threadIdx.x; i < wq; i += THREADS) qo[i] = from_f32<T>(sm[i] * iq * a.q_weight[i] * temp);
   if (!a.slots) return;
   const int slot = a.slots[t];
   const int page = slot / a.page_size, off = slot - page * a.page_size;
   T* kc = (T*)a.k_cache;
   T* vc = (T*)a.v_cache;
-  for (int i = threadIdx.x; i < wk; i += 256) {
+  for (int i = threadIdx.x; i < wk; i += THREADS) {
     const int h = i / a.d, e = i - h * a.d;
     const size_t head = (size_t)page * a.nkv + h;
     kc[(head * a.page_size + off) * a.d + e] = from_f32<T>(sm[wq + i] * ik * a.k_weight[i]);
@@ -73,9 +86,14 @@ extern "C" int qrt_qk_joint_norm_store(const JointNormArgs* args, int dtype, int
   QRT_CHECK(smem <= 64 * 1024, "qk_joint_norm_store: a token's %d query and key elements do not fit the block's memory",
             (a.nq + a.nkv) * a.d);
   if (num_tokens == 0) return 0;
-  if (dtype == QRT_F32) joint_norm_kernel<float><<<num_tokens, 256, smem, stream>>>(a);
-  else if (dtype == QRT_BF16) joint_norm_kernel<bf16_t><<<num_tokens, 256, smem, stream>>>(a);
-  else return qrt_fail("qk_joint_norm_store: unknown dtype %d", dtype);
+  const bool few = num_tokens <= 256;
+  if (dtype == QRT_F32) {
+    if (few) joint_norm_kernel<float, 1024><<<num_tokens, 1024, smem, stream>>>(a);
+    else joint_norm_kernel<float, 256><<<num_tokens, 256, smem, stream>>>(a);
+  } else if (dtype == QRT_BF16) {
+    if (few) joint_norm_kernel<bf16_t, 1024><<<num_tokens, 1024, smem, stream>>>(a);
+    else joint_norm_kernel<bf16_t, 256><<<num_tokens, 256, smem, stream>>>(a);
+  } else return qrt_fail("qk_joint_norm_store: unknown dtype %d", dtype);
   QRT_LAUNCH_CHECK("qk_joint_norm_store");
   return 0;
 }

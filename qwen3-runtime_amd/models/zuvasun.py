@@ -133,6 +133,30 @@ PRESETS: dict[str, ZuvasunConfig] = {
 PRESET_PAGE_SIZE = {"zuvasun_tiny_a": 16, "zuvasun_tiny_b": 8}
 
 
+def sized(width: int, layers: int, heads: int, kv_heads: int, dim: int, vocab: int, *, expert_ff: int, experts: int = 16,
+          top: int = 2, window: int = 2048, kv_rank: int = 384, rot_dim: int = 64) -> ZuvasunConfig:
+    """A configuration of the sizes of a real model, for measurements: a latent layer, a latent layer
+    that reads the first one's cache, and two layers whose values are their keys, in turn; a
+    mixture in every layer."""
+    rot = PairRotation(rot_dim, 1e6, _STRETCH(4.0, 4096, 32.0, 1.0))
+    own = SharedLatentSizes(heads, dim, rot_dim, dim, kv_rank, (dim + rot_dim) ** -0.5, rot, window)
+    att = KeyValueSizes(heads, kv_heads, dim, dim ** -0.5, 0.1, 1024)
+    ff = MixtureSizes(expert_ff, experts, top, 1.0)
+    out = []
+    for i in range(layers):
+        if i % 4 == 1:
+            out.append(ZuvasunLayer("latent_attention", SharedLatentSizes(heads, dim, rot_dim, dim, kv_rank, own.scale, rot, window,
+                                                                          kv_from=i - 1), ff))
+        else:
+            out.append(ZuvasunLayer("latent_attention" if i % 4 == 0 else "attention", own if i % 4 == 0 else att, ff))
+    return ZuvasunConfig(vocab=vocab, width=width, eps=1e-5, layers=tuple(out))
+
+
 register_architecture(ZuvasunConfig.architecture, ZuvasunConfig.from_dict, plan_zuvasun)
 for _name, _cfg in PRESETS.items():
     register_preset(_name, _cfg.to_dict(), PRESET_PAGE_SIZE.get(_name, 16))
+# layers of the sizes of the 4B and 8B dense presets, and of a smaller width, with a mixture like
+# `roserax_4b`'s in every layer, for measurements beside it
+register_preset("zuvasun_4b", sized(2560, 36, 32, 8, 128, 151936, expert_ff=1536).to_dict(), 16)
+register_preset("zuvasun_8b", sized(4096, 36, 32, 8, 128, 151936, expert_ff=2048, kv_rank=448).to_dict(), 16)
+register_preset("zuvasun_2b", sized(2048, 28, 16, 4, 128, 151936, expert_ff=1024, kv_rank=256).to_dict(), 16)
