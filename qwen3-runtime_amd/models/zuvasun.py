@@ -138,7 +138,7 @@ def sized(width: int, layers: int, heads: int, kv_heads: int, dim: int, vocab: i
     """A configuration of the sizes of a real model, for measurements: a latent layer, a latent layer
     that reads the first one's cache, and two layers whose values are their keys, in turn; a
     mixture in every layer."""
-    rot = PairRotation(rot_dim, 1e6, _STRETCH(4.0, 4096, 32.0, 1.0))
+    rot = PairRotation(rot_dim, 1e6, _STRETCH(8.0, 4096, 16.0, 1.0))
     own = SharedLatentSizes(heads, dim, rot_dim, dim, kv_rank, (dim + rot_dim) ** -0.5, rot, window)
     att = KeyValueSizes(heads, kv_heads, dim, dim ** -0.5, 0.1, 1024)
     ff = MixtureSizes(expert_ff, experts, top, 1.0)
