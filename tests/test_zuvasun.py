@@ -701,57 +701,44 @@ def test_greedy_generation_through_the_entry_point(folder, name, dtype, graphs):
 
 
 def test_greedy_generation_on_the_host(folder):
-    """The engine's own scheduler and sampler over the plain torch ops: requests of unequal lengths
-    under a small token budget, more of them than run at once."""
-    from qwen3_runtime_amd.engine.engine import Engine
-    from qwen3_runtime_amd.engine.request import Request  # noqa: F401  (the engine's own request type)
+    """The engine's own scheduler (admission, portions under a small token budget, two requests at
+    a time of three) and step function over the plain torch ops; the greedy choice is made here,
+    the sampler being a kernel."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.batch import StepEntry
+    from qwen3_runtime_amd.engine.request import Request
+    from qwen3_runtime_amd.engine.scheduler import Scheduler
 
     raw, page = config_d()
     cfg, w = P.load(folder("d"))
     loaded = load(folder("d"), page, 32, ("cpu", "float32"), max_seqs=2)
     prompts = list(traces.make_requests(raw["vocab"], [12, 3, 30], seed=4).values())
-    outs = generate_on_host(loaded, prompts, 16)
-    for prompt, tokens in zip(prompts, outs):
-        assert len(tokens) == 16
-        ref = P.forward(cfg, w, list(prompt) + tokens)[len(prompt) - 1: -1]
-        below = ref.max(-1).values - ref[range(16), tokens]
-        assert float(below.max()) < 1e-3
-
-
-def generate_on_host(loaded, prompts, max_tokens):
-    """Greedy tokens through the scheduler's plans and the step function, the choice made on the host."""
-    from qwen3_runtime_amd.engine.batch import StepEntry
-
-    tokens = [[] for _ in prompts]
-    fed = [0] * len(prompts)
-    live, waiting = [], list(range(len(prompts)))
-    while live or waiting:
-        while waiting and len(live) < 2:
-            i = waiting.pop(0)
-            loaded.cache.admit(f"r{i}")
-            live.append(i)
-        entries, who = [], []
-        budget = 10
-        for i in live:
-            have = list(prompts[i]) + tokens[i]
-            n = min(len(have) - fed[i], budget)
-            if n <= 0:
-                continue
-            budget -= n
-            last = fed[i] + n == len(have)
-            entries.append(StepEntry(f"r{i}", have[fed[i]: fed[i] + n], [n - 1] if last else []))
-            who.append((i, n, last))
+    engine = EngineConfig(page_size=page, num_pages=32, max_num_seqs=2, max_num_batched_tokens=10, dtype="float32", device="cpu")
+    scheduler = Scheduler(engine, loaded.cache, 100_000)
+    lengths = [16, 9, 16]  # the second ends first, and the third one's prompt is read beside the first one's decoding
+    requests = [Request(list(p), max_tokens=n) for p, n in zip(prompts, lengths)]
+    for r in requests:
+        scheduler.add(r)
+    sizes = set()
+    while not scheduler.is_finished():
+        batch = scheduler.schedule()
+        entries, caught = [], []
+        for r in batch:
+            at = loaded.cache.length(r.request_id)
+            upto = at + r.grant
+            caught.append(upto >= len(r.token_ids))
+            entries.append(StepEntry(r.request_id, r.token_ids[at:upto], [r.grant - 1] if caught[-1] else []))
+        sizes.add(tuple(sorted(r.grant for r in batch)))
         logits = loaded.runner.step(entries)
-        row = 0
-        for i, n, last in who:
-            fed[i] += n
-            if last:
-                tokens[i].append(int(logits[row].argmax()))
-                row += 1
-                if len(tokens[i]) == max_tokens:
-                    loaded.cache.release(f"r{i}")
-                    live.remove(i)
-    return tokens
+        rows = iter(logits if logits is not None else [])
+        scheduler.settle(batch, [int(next(rows).argmax()) if c else None for c in caught])
+    assert any(len(x) == 2 and x[0] == 1 and x[1] > 1 for x in sizes)  # a decoded token beside a prompt's portion
+    for prompt, r, n in zip(prompts, requests, lengths):
+        tokens = list(r.output_tokens)
+        assert len(tokens) == n
+        ref = P.forward(cfg, w, list(prompt) + tokens)[len(prompt) - 1: -1]
+        below = ref.max(-1).values - ref[range(n), tokens]
+        assert float(below.max()) < 1e-3
 
 
 @pytest.mark.gpu
