@@ -110,7 +110,7 @@ class _JointNormArgs(Structure):
         ("qk", c_void_p), ("row", c_long), ("bias", c_void_p), ("q_weight", c_void_p), ("k_weight", c_void_p),
         ("positions", c_void_p), ("q_out", c_void_p), ("slots", c_void_p), ("k_cache", c_void_p), ("v_cache", c_void_p),
         ("page_size", c_int), ("nq", c_int), ("nkv", c_int), ("d", c_int), ("values_are_keys", c_int),
-        ("eps", c_float), ("temp_coef", c_float), ("temp_every", c_int),
+        ("eps", c_float), ("temp_coef", c_float), ("temp_every", c_int), ("num_tokens", c_int), ("group_values", c_int), ("wide", c_int),
     ]
 
 

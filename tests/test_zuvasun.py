@@ -300,6 +300,10 @@ def test_values_are_the_keys(backend, nq, nkv, d, temp, page):
     # the pages are used again, token by token from the start
     driver = MixerDriver(mixer, device, dt, ops, page, -(-100 // page))
     assert_rows(driver.run("c", h[0][:100], in_steps(100, (1,))), want[0][:100], dtype, "one by one")
+    # long portions, whose values are stored eight tokens at a time: from a page's start, and from its third place
+    for cuts in ([(0, t)], [(0, 3), (3, 300), (303, t - 303)]):
+        driver = MixerDriver(mixer, device, dt, ops, page, -(-t // page))
+        assert_rows(driver.run("d", h[0], cuts), want[0], dtype, f"portions {cuts}")
 
 
 def test_attention_options_that_do_not_go_together():
